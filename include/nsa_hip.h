@@ -1,0 +1,56 @@
+/*
+ * C ABI of libnsa_hip.so - hand-written gfx950 (MI355X) kernels for the Native Sparse
+ * Attention operator path.  Every entry point replaces one Triton launch site (or one
+ * torch-op chain) of the reference's native_sparse_attention/ops package; the citation
+ * on each declaration names that site.
+ *
+ * Conventions
+ *  - All pointers are device pointers owned by the caller.  The library never allocates,
+ *    frees, retains or synchronises; work is enqueued on `stream` (a hipStream_t).
+ *  - dtype: NSA_BF16 or NSA_FP16 for q/k/v/x/w/o tensors; accumulation is fp32.
+ *  - Strides are in elements; the innermost (head_dim) stride must be 1.
+ *  - Varlen tensors are [total_len, heads, head_dim]; cu_seqlens is int32 [batch+1].
+ *  - Return value: NSA_OK (0) or a negative NSA_ERR_* code; nothing is launched on error.
+ *  - Re-entrant: no global state.
+ */
+#ifndef NSA_HIP_H
+#define NSA_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NSA_OK 0
+#define NSA_ERR_BAD_ARG (-1)      /* null pointer, negative size, inconsistent shapes   */
+#define NSA_ERR_UNSUPPORTED (-2)  /* head_dim / block_size / dtype outside the built set */
+#define NSA_ERR_WORKSPACE (-3)    /* workspace_bytes smaller than nsa_*_workspace_bytes  */
+#define NSA_ERR_LAUNCH (-4)       /* hipGetLastError() after the launch was not success  */
+
+#define NSA_BF16 0
+#define NSA_FP16 1
+
+/* Library version (major*10000 + minor*100 + patch). */
+int nsa_version(void);
+
+/* ---- topk_sparse_attention -------------------------------------------------------------
+ * Forward: replaces forward_kernel launched from _topk_sparse_attention_fwd
+ * (native_sparse_attention/ops/triton/topk_sparse_attention.py:828-909).
+ *   q,o [T,Hq,D]; k,v [T,Hkv,D]; topk_idx int32 [Hkv,T,topk] (entries <0 or beyond the
+ *   query's own block are skipped); lse fp32 [Hq,T] in base-2 units (contiguous).
+ * workspace holds a block-transposed copy of V: nsa_topk_attn_fwd_workspace_bytes().
+ */
+size_t nsa_topk_attn_fwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t head_dim);
+int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t* topk_idx, void* o, float* lse,
+                      const int32_t* cu_seqlens, int64_t total_len, int64_t batch, int64_t num_q_heads,
+                      int64_t num_kv_heads, int64_t head_dim, int64_t topk, int64_t block_size, int64_t q_stride_n,
+                      int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n,
+                      int64_t v_stride_h, int64_t idx_stride_h, int64_t idx_stride_n, int64_t idx_stride_k,
+                      int64_t o_stride_n, int64_t o_stride_h, float sm_scale, int dtype, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NSA_HIP_H */

@@ -1,0 +1,87 @@
+// Shared device/host helpers for the gfx950 NSA kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nsa_hip.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define NSA_LOG2E 1.4426950408889634f
+
+// Element-type traits: 8-wide register fragments and the 16x16x32 / 32x32x16 MFMA for that type.
+// Fragment layout (wave64): A is [16][32] with lane l holding row l%16, k = 8*(l/16)..+7;
+// B is [32][16] with lane l holding column l%16, k = 8*(l/16)..+7; the 16x16 result has lane l
+// holding column l%16, rows 4*(l/16)..+3.
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  using v8 = bf16x8;
+  using v4 = bf16x4;
+  static __device__ __forceinline__ f32x4 mfma16(v8 a, v8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Elem<_Float16> {
+  using v8 = f16x8;
+  using v4 = f16x4;
+  static __device__ __forceinline__ f32x4 mfma16(v8 a, v8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename V> __device__ __forceinline__ V ld16(const void* p) {
+  static_assert(sizeof(V) == 16, "16-byte fragment");
+  uint4 r = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(V, r);
+}
+template <typename V> __device__ __forceinline__ V zero16() {
+  uint4 z = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(V, z);
+}
+template <typename V> __device__ __forceinline__ void st16(void* p, V v) {
+  *reinterpret_cast<uint4*>(p) = __builtin_bit_cast(uint4, v);
+}
+template <typename V> __device__ __forceinline__ void st8(void* p, V v) {
+  static_assert(sizeof(V) == 8, "8-byte fragment");
+  *reinterpret_cast<uint2*>(p) = __builtin_bit_cast(uint2, v);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Index of the sequence that holds global token t: largest b with cu[b] <= t.
+__device__ __forceinline__ int find_sequence(const int32_t* __restrict__ cu, int batch, int t) {
+  int lo = 0, hi = batch;  // invariant: cu[lo] <= t < cu[hi]
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// Spread consecutive logical work ids over the 8 XCDs in contiguous runs: hardware hands
+// workgroup i to XCD i%8, so logical id = (i%8)*ceil(n/8) + i/8 keeps neighbours on one L2.
+__device__ __forceinline__ long long xcd_remap(long long wg, long long n_wg) {
+  long long per = (n_wg + 7) / 8;
+  return (wg % 8) * per + wg / 8;
+}
+
+static inline int nsa_check_launch() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? NSA_OK : NSA_ERR_LAUNCH;
+}
+
+// Number of 32-key chunk slots in a block-transposed copy of a [T, H, D] tensor: every
+// sequence starts on a fresh slot, so at most one slot of slack per sequence boundary.
+static inline int64_t nsa_chunk_slots(int64_t total_len, int64_t batch) { return (total_len + 31) / 32 + batch + 1; }

@@ -1,0 +1,193 @@
+// Forward of block-sparse GQA attention (topk_sparse_attention).
+//
+// One wavefront owns one (token, kv-head) pair and the up-to-16 query heads of that GQA
+// group.  Scores are produced transposed, S^T[key][head] = K * Q^T, so that each lane ends
+// up holding values of a single head: the row maximum and sum become per-lane scalars plus
+// two cross-lane steps, and P^T is already in the B-operand layout of the next MFMA,
+// O^T[d][head] += V^T[d][key] * P^T[key][head].  K rows are read straight from global memory
+// in A-operand layout (16 bytes per lane); V comes from the block-transposed copy built by
+// block_transpose_kernel.  Nothing is staged in LDS: with one token per wave every K/V
+// element feeds exactly one MFMA, so there is no reuse for LDS to exploit.
+#include "block_transpose.h"
+
+struct TopkFwdParams {
+  const void* q; const void* k; const void* vt; const int32_t* idx; void* o; float* lse; const int32_t* cu;
+  int total_len, batch, Hkv, G, GT, topk, n_slots;
+  long long n_items;
+  long long qsn, qsh, ksn, ksh, ish, isn, isk, osn, osh;
+  float qk_scale;  // sm_scale * log2(e)
+};
+
+template <typename T, int D, int BS>
+__global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  using v4 = typename E::v4;
+  constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16, NCH = BS / 32;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 15, lg = lane >> 4;
+  const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
+  if (item >= p.n_items) return;
+  const int t = (int)(item % p.total_len);
+  const int gt = (int)((item / p.total_len) % p.GT);
+  const int h = (int)(item / ((long long)p.total_len * p.GT));
+  const int b = find_sequence(p.cu, p.batch, t);
+  const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
+  const int pos = t - s0, qb = pos / BS;
+  const int slot0 = seq_first_slot(p.cu, b);
+
+  const int hq = gt * 16 + li;
+  const bool has_head = hq < p.G;
+  const T* qp = (const T*)p.q + (long long)t * p.qsn + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
+  v8 qf[NK];
+#pragma unroll
+  for (int kk = 0; kk < NK; kk++) qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+
+  f32x4 acc[NDT];
+#pragma unroll
+  for (int i = 0; i < NDT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+
+  const int32_t* ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
+  const T* kbase = (const T*)p.k + (long long)s0 * p.ksn + (long long)h * p.ksh + 8 * lg;
+  const T* vbase = (const T*)p.vt + ((long long)h * p.n_slots + slot0) * D * 32 + li * 32 + 8 * lg;
+
+  for (int e = 0; e < p.topk; e++) {
+    const int blk = ip[(long long)e * p.isk];
+    if (blk < 0 || blk > qb) continue;
+    const int key0 = blk * BS;
+    f32x4 s[NSUB];
+#pragma unroll
+    for (int nt = 0; nt < NSUB; nt++) {
+      int row = key0 + 16 * nt + li;
+      row = row < len ? row : len - 1;
+      const T* kp = kbase + (long long)row * p.ksn;
+      f32x4 c = {0.f, 0.f, 0.f, 0.f};
+      if (key0 + 16 * nt <= pos) {  // wave-uniform: sub-tiles wholly in the future are never loaded
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) c = E::mfma16(ld16<v8>(kp + 32 * kk), qf[kk], c);
+      }
+      s[nt] = c;
+    }
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < NSUB; nt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        int key = key0 + 16 * nt + 4 * lg + r;
+        float x = key <= pos ? s[nt][r] * p.qk_scale : -INFINITY;
+        s[nt][r] = x;
+        mloc = fmaxf(mloc, x);
+      }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    const float m_new = fmaxf(m, mloc);  // finite: key0 <= pos is always visible
+    const float alpha = fast_exp2(m - m_new);
+    m = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < NSUB; nt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        float x = fast_exp2(s[nt][r] - m_new);
+        s[nt][r] = x;
+        psum += x;
+      }
+    lsum = lsum * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < NDT; i++) acc[i] *= alpha;
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+      if (key0 + 32 * c > pos) break;  // wholly masked chunk: its slot of the transposed copy may not exist
+      v8 pf;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        pf[r] = (T)s[2 * c][r];
+        pf[4 + r] = (T)s[2 * c + 1][r];
+      }
+      const T* vp = vbase + (long long)((key0 >> 5) + c) * D * 32;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) acc[dt] = E::mfma16(ld16<v8>(vp + dt * 16 * 32), pf, acc[dt]);
+    }
+  }
+  lsum += __shfl_xor(lsum, 16);
+  lsum += __shfl_xor(lsum, 32);
+  const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+  if (has_head) {
+    T* op = (T*)p.o + (long long)t * p.osn + (long long)(h * p.G + hq) * p.osh + 4 * lg;
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) {
+      v4 out;
+#pragma unroll
+      for (int r = 0; r < 4; r++) out[r] = (T)(acc[dt][r] * inv);
+      st8(op + 16 * dt, out);
+    }
+    if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + t] = lsum > 0.f ? m + fast_log2(lsum) : -INFINITY;
+  }
+}
+
+template <typename T, int D, int BS>
+static int launch_fwd(const TopkFwdParams& p, const void* v, long long vsn, long long vsh, hipStream_t stream) {
+  launch_block_transpose<T, D>((const T*)v, (T*)p.vt, p.cu, p.batch, vsn, vsh, p.n_slots, p.Hkv, stream);
+  long long n_wg = (p.n_items + 3) / 4;
+  n_wg = (n_wg + 7) / 8 * 8;
+  topk_fwd_kernel<T, D, BS><<<dim3((unsigned)n_wg), 256, 0, stream>>>(p);
+  return nsa_check_launch();
+}
+
+template <typename T, int D>
+static int dispatch_bs(int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, hipStream_t s) {
+  switch (bs) {
+    case 32: return launch_fwd<T, D, 32>(p, v, vsn, vsh, s);
+    case 64: return launch_fwd<T, D, 64>(p, v, vsn, vsh, s);
+    case 128: return launch_fwd<T, D, 128>(p, v, vsn, vsh, s);
+    case 256: return launch_fwd<T, D, 256>(p, v, vsn, vsh, s);
+  }
+  return NSA_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+static int dispatch_d(int d, int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, hipStream_t s) {
+  switch (d) {
+    case 32: return dispatch_bs<T, 32>(bs, p, v, vsn, vsh, s);
+    case 64: return dispatch_bs<T, 64>(bs, p, v, vsn, vsh, s);
+    case 96: return dispatch_bs<T, 96>(bs, p, v, vsn, vsh, s);
+    case 128: return dispatch_bs<T, 128>(bs, p, v, vsn, vsh, s);
+  }
+  return NSA_ERR_UNSUPPORTED;
+}
+
+extern "C" size_t nsa_topk_attn_fwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t head_dim) {
+  return (size_t)num_kv_heads * (size_t)nsa_chunk_slots(total_len, batch) * (size_t)head_dim * 32 * 2;
+}
+
+extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t* topk_idx, void* o, float* lse,
+                                 const int32_t* cu_seqlens, int64_t total_len, int64_t batch, int64_t num_q_heads,
+                                 int64_t num_kv_heads, int64_t head_dim, int64_t topk, int64_t block_size,
+                                 int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                                 int64_t v_stride_n, int64_t v_stride_h, int64_t idx_stride_h, int64_t idx_stride_n,
+                                 int64_t idx_stride_k, int64_t o_stride_n, int64_t o_stride_h, float sm_scale, int dtype,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  if (!q || !k || !v || !topk_idx || !o || !lse || !cu_seqlens || !workspace) return NSA_ERR_BAD_ARG;
+  if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
+  if (total_len >= (1ll << 31)) return NSA_ERR_BAD_ARG;
+  // 16-byte fragment loads need 8-element alignment of every row start
+  if ((q_stride_n | q_stride_h | k_stride_n | k_stride_h | v_stride_n | v_stride_h) % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  if ((o_stride_n | o_stride_h) % 4 != 0) return NSA_ERR_UNSUPPORTED;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)workspace) % 16 != 0 || (uintptr_t)o % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_topk_attn_fwd_workspace_bytes(total_len, batch, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
+  TopkFwdParams p;
+  p.q = q; p.k = k; p.vt = workspace; p.idx = topk_idx; p.o = o; p.lse = lse; p.cu = cu_seqlens;
+  p.total_len = (int)total_len; p.batch = (int)batch; p.Hkv = (int)num_kv_heads; p.G = (int)(num_q_heads / num_kv_heads);
+  p.GT = (p.G + 15) / 16; p.topk = (int)topk; p.n_slots = (int)nsa_chunk_slots(total_len, batch);
+  p.n_items = (long long)total_len * p.GT * p.Hkv;
+  p.qsn = q_stride_n; p.qsh = q_stride_h; p.ksn = k_stride_n; p.ksh = k_stride_h;
+  p.ish = idx_stride_h; p.isn = idx_stride_n; p.isk = idx_stride_k; p.osn = o_stride_n; p.osh = o_stride_h;
+  p.qk_scale = sm_scale * NSA_LOG2E;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, s);
+  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, s);
+  return NSA_ERR_UNSUPPORTED;
+}
+
+extern "C" int nsa_version(void) { return 100; }

@@ -1,0 +1,68 @@
+"""ctypes binding of libnsa_hip.so (declared in include/nsa_hip.h).
+
+The shared library is the only compute path: if it has not been built the first call raises;
+there is no PyTorch fallback.
+"""
+import ctypes
+import os
+from ctypes import c_float, c_int, c_int64, c_size_t, c_void_p
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libnsa_hip.so")
+_lib = None
+
+NSA_BF16, NSA_FP16 = 0, 1
+_ERR = {-1: "bad argument", -2: "unsupported shape/dtype/alignment", -3: "workspace too small", -4: "kernel launch failed"}
+
+P, I, F, Z = c_void_p, c_int64, c_float, c_size_t
+_SIGNATURES = {
+    "nsa_version": (c_int, []),
+    "nsa_topk_attn_fwd_workspace_bytes": (Z, [I, I, I, I]),
+    "nsa_topk_attn_fwd": (c_int, [P] * 7 + [I] * 7 + [I] * 11 + [F, c_int, P, Z, P]),
+}
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                "libnsa_hip.so is not built (%s missing): run `python native-sparse-attention-triton_amd/build.py`" % _LIB_PATH
+            )
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def check(code: int, what: str):
+    if code != 0:
+        raise RuntimeError("%s failed: %s (code %d)" % (what, _ERR.get(code, "unknown"), code))
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return NSA_BF16
+    if t.dtype == torch.float16:
+        return NSA_FP16
+    raise AssertionError("bf16 or fp16 expected, got %s" % t.dtype)
+
+
+def stream_ptr(t: torch.Tensor):
+    assert t.is_cuda, "the HIP kernels need device tensors"
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)

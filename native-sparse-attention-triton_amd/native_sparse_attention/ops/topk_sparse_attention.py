@@ -1,0 +1,87 @@
+"""topk_sparse_attention: same signature and checks as the reference operator
+(native_sparse_attention/ops/triton/topk_sparse_attention.py:1112-1217), running on the gfx950 kernels."""
+import math
+from typing import Optional
+
+import torch
+
+from .. import _lib
+
+
+def _last_dim_contiguous(t: torch.Tensor) -> torch.Tensor:
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _topk_sparse_attention_fwd(q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale):
+    """Returns (o [T,Hq,D], lse fp32 [Hq,T] in base-2 units); mirrors _topk_sparse_attention_fwd (:828-909)."""
+    assert k.dtype == q.dtype and v.dtype == q.dtype
+    assert cu_seqlens_q.dtype == torch.int32 and cu_seqlens_k.dtype == torch.int32
+    assert block_size in {32, 64, 128, 256}
+    q_len, num_q_heads, head_dim = q.shape
+    k_len, num_k_heads, _ = k.shape
+    v_len, num_v_heads, _ = v.shape
+    batch = cu_seqlens_q.shape[0] - 1
+    assert q_len == k_len and k_len == v_len
+    topk = topk_idx.shape[-1]
+    assert topk_idx.shape[0] == num_k_heads and topk_idx.shape[1] == q_len
+    assert num_k_heads == num_v_heads and num_q_heads % num_k_heads == 0
+    q, k, v = map(_last_dim_contiguous, (q, k, v))
+    o = torch.empty((q_len, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+    lse = torch.empty((num_q_heads, q_len), dtype=torch.float32, device=q.device)
+    lib = _lib.load()
+    ws = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(q_len, batch, num_k_heads, head_dim), q.device)
+    rc = lib.nsa_topk_attn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), topk_idx.data_ptr(), o.data_ptr(), lse.data_ptr(),
+        cu_seqlens_q.data_ptr(), q_len, batch, num_q_heads, num_k_heads, head_dim, topk, block_size,
+        q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+        topk_idx.stride(0), topk_idx.stride(1), topk_idx.stride(2), o.stride(0), o.stride(1),
+        sm_scale, _lib.dtype_code(q), ws.data_ptr(), ws.numel(), _lib.stream_ptr(q),
+    )
+    _lib.check(rc, "nsa_topk_attn_fwd")
+    return o, lse
+
+
+class TopkSparseAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale=None):
+        assert q.dtype == torch.bfloat16 or q.dtype == torch.float16
+        assert q.dtype == k.dtype and k.dtype == v.dtype
+        assert topk_idx.dtype == torch.int32
+        assert cu_seqlens_q.dtype == torch.int32 and cu_seqlens_k.dtype == torch.int32
+        if sm_scale is None:
+            sm_scale = 1 / math.sqrt(q.shape[-1])
+        o, lse = _topk_sparse_attention_fwd(
+            q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale)
+        ctx.save_for_backward(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, topk_idx)
+        ctx.sm_scale, ctx.block_size = sm_scale, block_size
+        ctx.max_seqlen_q, ctx.max_seqlen_k = max_seqlen_q, max_seqlen_k
+        return o
+
+    @staticmethod
+    def backward(ctx, do, *args):
+        raise NotImplementedError("backward kernels are not built yet")
+
+
+def topk_sparse_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    topk_idx: torch.Tensor,
+    block_size: int,
+    cu_seqlens: torch.Tensor,
+    softmax_scale: Optional[float] = None,
+) -> torch.Tensor:
+    """Block-sparse GQA attention, varlen layout.
+
+    Args:
+        q: [total_len, num_q_heads, head_dim]; k, v: [total_len, num_kv_heads, head_dim] (bf16/fp16)
+        topk_idx: int32 [num_kv_heads, total_len, topk], per-sequence block ids, -1 = padding
+        block_size: key/value block size (32, 64, 128 or 256)
+        cu_seqlens: int32 [batch + 1]
+        softmax_scale: defaults to 1/sqrt(head_dim)
+    Returns: [total_len, num_q_heads, head_dim]
+
+    The kernels walk the token range directly, so unlike the reference wrapper (:1205) no
+    host synchronisation is needed to learn the longest sequence.
+    """
+    return TopkSparseAttention.apply(q, k, v, topk_idx, block_size, cu_seqlens, cu_seqlens, None, None, softmax_scale)
