@@ -50,6 +50,28 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
                       int64_t o_stride_n, int64_t o_stride_h, float sm_scale, int dtype, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* Backward: replaces backward_sum_o_do, count_query + reorder_topk_idx (with their host
+ * synchronisations and argsort), backward_dkdv and backward_dq launched from
+ * _topk_sparse_attention_bwd (native_sparse_attention/ops/triton/topk_sparse_attention.py:912-1109).
+ *   o,dout,dq [T,Hq,D]; dk,dv [T,Hkv,D]; lse as produced by nsa_topk_attn_fwd.
+ *   strides: HOST array of 19 element strides in the order
+ *     q(n,h) k(n,h) v(n,h) o(n,h) dout(n,h) idx(h,n,k) dq(n,h) dk(n,h) dv(n,h).
+ *   out_segment_offsets / out_queries: optional (both or neither) device buffers that
+ *   receive the "KV block -> queries" reverse index built on the way:
+ *     segments = nsa_topk_reverse_index_segments(); segment s = kv_head*(T/block+batch) + global block;
+ *     out_segment_offsets int32 [segments+1]; out_queries int32 [Hkv*T*topk], the tokens of
+ *     segment s are out_queries[off[s] : off[s+1]], ascending.
+ * dK/dV are reduced in a fixed order (no atomics): results are run-to-run deterministic.
+ */
+size_t nsa_topk_attn_bwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                         int64_t head_dim, int64_t topk, int64_t block_size);
+int64_t nsa_topk_reverse_index_segments(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t block_size);
+int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
+                      const int32_t* topk_idx, const int32_t* cu_seqlens, void* dq, void* dk, void* dv, int64_t total_len,
+                      int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t topk,
+                      int64_t block_size, const int64_t* strides, float sm_scale, int dtype, void* workspace,
+                      size_t workspace_bytes, int32_t* out_segment_offsets, int32_t* out_queries, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,9 @@ _SIGNATURES = {
     "nsa_version": (c_int, []),
     "nsa_topk_attn_fwd_workspace_bytes": (Z, [I, I, I, I]),
     "nsa_topk_attn_fwd": (c_int, [P] * 7 + [I] * 7 + [I] * 11 + [F, c_int, P, Z, P]),
+    "nsa_topk_attn_bwd_workspace_bytes": (Z, [I] * 7),
+    "nsa_topk_reverse_index_segments": (I, [I] * 4),
+    "nsa_topk_attn_bwd": (c_int, [P] * 11 + [I] * 7 + [P, F, c_int, P, Z, P, P, P]),
 }
 
 
@@ -62,6 +65,11 @@ def dtype_code(t: torch.Tensor) -> int:
 def stream_ptr(t: torch.Tensor):
     assert t.is_cuda, "the HIP kernels need device tensors"
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def host_i64(values):
+    """Host int64 array for the entry points that take their strides as one array."""
+    return (c_int64 * len(values))(*[int(v) for v in values])
 
 
 def workspace(nbytes: int, device) -> torch.Tensor:

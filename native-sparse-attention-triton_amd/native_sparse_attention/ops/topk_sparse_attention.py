@@ -41,6 +41,43 @@ def _topk_sparse_attention_fwd(q, k, v, topk_idx, block_size, cu_seqlens_q, cu_s
     return o, lse
 
 
+def _topk_sparse_attention_bwd(o, do, lse, q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k,
+                               max_seqlen_q, max_seqlen_k, sm_scale, return_reverse_index=False):
+    """Returns (dq, dk, dv); mirrors _topk_sparse_attention_bwd (:912-1109)."""
+    assert block_size in {32, 64, 128, 256}
+    q_len, num_q_heads, head_dim = q.shape
+    num_k_heads = k.shape[1]
+    batch = cu_seqlens_q.shape[0] - 1
+    topk = topk_idx.shape[-1]
+    q, k, v, o, do = map(_last_dim_contiguous, (q, k, v, o, do))
+    dq = torch.empty((q_len, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+    dk = torch.empty((q_len, num_k_heads, head_dim), dtype=q.dtype, device=q.device)
+    dv = torch.empty((q_len, num_k_heads, head_dim), dtype=q.dtype, device=q.device)
+    lib = _lib.load()
+    ws = _lib.workspace(
+        lib.nsa_topk_attn_bwd_workspace_bytes(q_len, batch, num_q_heads, num_k_heads, head_dim, topk, block_size), q.device)
+    strides = _lib.host_i64(
+        [q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), o.stride(0), o.stride(1),
+         do.stride(0), do.stride(1), topk_idx.stride(0), topk_idx.stride(1), topk_idx.stride(2),
+         dq.stride(0), dq.stride(1), dk.stride(0), dk.stride(1), dv.stride(0), dv.stride(1)])
+    seg_off = queries = None
+    if return_reverse_index:
+        n_seg = lib.nsa_topk_reverse_index_segments(q_len, batch, num_k_heads, block_size)
+        seg_off = torch.empty(n_seg + 1, dtype=torch.int32, device=q.device)
+        queries = torch.empty(num_k_heads * q_len * topk, dtype=torch.int32, device=q.device)
+    rc = lib.nsa_topk_attn_bwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(), topk_idx.data_ptr(),
+        cu_seqlens_q.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), q_len, batch, num_q_heads, num_k_heads,
+        head_dim, topk, block_size, strides, sm_scale, _lib.dtype_code(q), ws.data_ptr(), ws.numel(),
+        seg_off.data_ptr() if return_reverse_index else None, queries.data_ptr() if return_reverse_index else None,
+        _lib.stream_ptr(q),
+    )
+    _lib.check(rc, "nsa_topk_attn_bwd")
+    if return_reverse_index:
+        return dq, dk, dv, seg_off, queries
+    return dq, dk, dv
+
+
 class TopkSparseAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale=None):
@@ -59,7 +96,11 @@ class TopkSparseAttention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, *args):
-        raise NotImplementedError("backward kernels are not built yet")
+        q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, topk_idx = ctx.saved_tensors
+        dq, dk, dv = _topk_sparse_attention_bwd(
+            o, do, lse, q, k, v, topk_idx, ctx.block_size, cu_seqlens_q, cu_seqlens_k,
+            ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.sm_scale)
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 def topk_sparse_attention(

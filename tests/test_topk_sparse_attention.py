@@ -68,3 +68,52 @@ def test_rejects_bad_dtypes(device):
         topk_sparse_attention(qb, qb[:, :1], qb[:, :1], idx.long(), 64, cu)   # idx must be int32
     with pytest.raises(AssertionError):
         topk_sparse_attention(qb, qb[:, :1], qb[:, :1], idx, 48, cu)          # block size set
+
+
+def _grad_check(device, lens, Hq, Hkv, d, bs, topk, dtype, local, seed=0):
+    q, k, v, cu = _make(lens, Hq, Hkv, d, dtype, device, seed)
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=1, local_blocks=local)
+    g = torch.Generator(device=device).manual_seed(9)
+    do = torch.randn(q.shape, generator=g, device=device).to(dtype)
+    q1, k1, v1 = (x.clone().requires_grad_() for x in (q, k, v))
+    o = topk_sparse_attention(q1, k1, v1, idx, bs, cu)
+    o.backward(do)
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, k, v))
+    want = oracle.topk_sparse_attention(qf, kf, vf, idx, bs, cu)
+    want.backward(do.float())
+    # gradients of early keys sum over thousands of queries: bound errors relative to the
+    # largest reference magnitude when that exceeds 1 (bf16 output rounding alone is 2^-9 relative)
+    for name, got, ref in (("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)):
+        assert_close(got, ref, name, rel_to=ref.abs().max().item())
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv,d,bs,topk,dtype,local", CASES)
+def test_backward_matches_oracle(device, lens, Hq, Hkv, d, bs, topk, dtype, local):
+    print("case", lens, Hq, Hkv, d, bs, topk, dtype, flush=True)
+    _grad_check(device, lens, Hq, Hkv, d, bs, topk, dtype, local)
+
+
+def test_reverse_index_bit_exact_and_deterministic(device):
+    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
+    lens, Hq, Hkv, d, bs, topk = [700, 64, 1500], 16, 2, 64, 64, 6
+    q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device)
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=4)
+    o, lse = _topk_sparse_attention_fwd(q, k, v, idx, bs, cu, cu, None, None, d ** -0.5)
+    do = torch.randn_like(o)
+    dq, dk, dv, seg_off, queries = _topk_sparse_attention_bwd(
+        o, do, lse, q, k, v, idx, bs, cu, cu, None, None, d ** -0.5, return_reverse_index=True)
+    cu_blk, offs, qs = oracle.build_reverse_index(idx.cpu().numpy(), cu.cpu().numpy(), bs)
+    T, B = int(cu[-1]), len(lens)
+    max_blocks = T // bs + B
+    seg_off, queries = seg_off.cpu().numpy(), queries.cpu().numpy()
+    total_blocks = int(cu_blk[-1])
+    for h in range(Hkv):
+        for g in range(total_blocks):
+            s = h * max_blocks + g
+            got = queries[seg_off[s]:seg_off[s + 1]].tolist()
+            assert got == qs[h, offs[h, g]:offs[h, g + 1]].tolist(), (h, g)
+        for g in range(total_blocks, max_blocks):                      # unused segments are empty
+            s = h * max_blocks + g
+            assert seg_off[s] == seg_off[s + 1]
+    dq2, dk2, dv2 = _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, None, None, d ** -0.5)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
