@@ -40,7 +40,12 @@ int nsa_version(void);
  *   q,o [T,Hq,D]; k,v [T,Hkv,D]; topk_idx int32 [Hkv,T,topk] (entries <0 or beyond the
  *   query's own block are skipped); lse fp32 [Hq,T] in base-2 units (contiguous).
  * workspace holds a block-transposed copy of V: nsa_topk_attn_fwd_workspace_bytes().
+ * phases: NSA_FWD_PHASE_ALL, or a subset when the caller re-uses the workspace of a previous
+ * call with the same V (profiling a single kernel).
  */
+#define NSA_FWD_PHASE_TRANSPOSE 1
+#define NSA_FWD_PHASE_ATTEND 2
+#define NSA_FWD_PHASE_ALL 3
 size_t nsa_topk_attn_fwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t head_dim);
 int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t* topk_idx, void* o, float* lse,
                       const int32_t* cu_seqlens, int64_t total_len, int64_t batch, int64_t num_q_heads,
@@ -48,7 +53,7 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
                       int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n,
                       int64_t v_stride_h, int64_t idx_stride_h, int64_t idx_stride_n, int64_t idx_stride_k,
                       int64_t o_stride_n, int64_t o_stride_h, float sm_scale, int dtype, void* workspace,
-                      size_t workspace_bytes, void* stream);
+                      size_t workspace_bytes, int phases, void* stream);
 
 /* Backward: replaces backward_sum_o_do, count_query + reorder_topk_idx (with their host
  * synchronisations and argsort), backward_dkdv and backward_dq launched from
@@ -62,7 +67,13 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
  *     out_segment_offsets int32 [segments+1]; out_queries int32 [Hkv*T*topk], the tokens of
  *     segment s are out_queries[off[s] : off[s+1]], ascending.
  * dK/dV are reduced in a fixed order (no atomics): results are run-to-run deterministic.
+ * phases: NSA_BWD_PHASE_ALL, or a subset to re-run single passes on a workspace that an
+ * earlier call with identical arguments has already filled (PREP = delta + reverse index).
  */
+#define NSA_BWD_PHASE_PREP 1
+#define NSA_BWD_PHASE_DKDV 2
+#define NSA_BWD_PHASE_DQ 4
+#define NSA_BWD_PHASE_ALL 7
 size_t nsa_topk_attn_bwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
                                          int64_t head_dim, int64_t topk, int64_t block_size);
 int64_t nsa_topk_reverse_index_segments(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t block_size);
@@ -70,7 +81,8 @@ int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, const void* o
                       const int32_t* topk_idx, const int32_t* cu_seqlens, void* dq, void* dk, void* dv, int64_t total_len,
                       int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t topk,
                       int64_t block_size, const int64_t* strides, float sm_scale, int dtype, void* workspace,
-                      size_t workspace_bytes, int32_t* out_segment_offsets, int32_t* out_queries, void* stream);
+                      size_t workspace_bytes, int32_t* out_segment_offsets, int32_t* out_queries, int phases,
+                      void* stream);
 
 #ifdef __cplusplus
 }

@@ -476,7 +476,7 @@ struct BwdArgs {
   const void *q, *k, *v, *o, *dout; const float* lse; const int32_t* idx; const int32_t* cu; void *dq, *dk, *dv;
   int64_t T, B, Hq, Hkv, D, topk, bs;
   int64_t qsn, qsh, ksn, ksh, vsn, vsh, osn, osh, dsn, dsh, ish, isn, isk, dqsn, dqsh, dksn, dksh, dvsn, dvsh;
-  float sm_scale; char* ws; hipStream_t stream;
+  float sm_scale; char* ws; hipStream_t stream; int phases;
   int32_t* out_seg_off; int32_t* out_queries;  // optional copies of the reverse index (tests)
 };
 
@@ -510,19 +510,21 @@ static int run_bwd(const BwdArgs& a) {
   float* delta = (float*)(ws + L.delta);
   const int G = (int)(a.Hq / a.Hkv), GT = (G + 15) / 16;
   const int n_seg = (int)(a.Hkv * L.max_blocks);
-  {
+  if (a.phases & NSA_BWD_PHASE_PREP) {
     constexpr int LPR = D / 8, LPR2 = LPR <= 4 ? 4 : (LPR <= 8 ? 8 : 16);
     const long long rows = (long long)a.T * a.Hq;
     delta_kernel<T, D><<<(unsigned)((rows + 256 / LPR2 - 1) / (256 / LPR2)), 256, 0, a.stream>>>(
         (const T*)a.o, (const T*)a.dout, delta, (int)a.T, (int)a.Hq, a.osn, a.osh, a.dsn, a.dsh);
   }
-  int rc = build_reverse_index(a, L);
-  if (rc != NSA_OK) return rc;
+  if (a.phases & NSA_BWD_PHASE_PREP) {
+    int rc = build_reverse_index(a, L);
+    if (rc != NSA_OK) return rc;
+  }
   if (a.out_seg_off) {
     (void)hipMemcpyAsync(a.out_seg_off, ws + L.seg_off, (size_t)(n_seg + 1) * 4, hipMemcpyDeviceToDevice, a.stream);
     (void)hipMemcpyAsync(a.out_queries, ws + L.vals_out, (size_t)L.n_pairs * 4, hipMemcpyDeviceToDevice, a.stream);
   }
-  {
+  if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;
     p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.cu = a.cu;
     p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_off = (const int32_t*)(ws + L.seg_off);
@@ -536,7 +538,7 @@ static int run_bwd(const BwdArgs& a) {
     dkdv_reduce_kernel<T, D, BS><<<(unsigned)n_seg, 256, 0, a.stream>>>(
         p.partial, p.chunk_off, a.cu, p.cu_blk, (int)a.B, (int)L.max_blocks, (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
   }
-  {
+  if (a.phases & NSA_BWD_PHASE_DQ) {
     T* kt = (T*)(ws + L.kt);
     launch_block_transpose<T, D>((const T*)a.k, kt, a.cu, a.B, a.ksn, a.ksh, L.n_slots, a.Hkv, a.stream);
     DqParams p;
@@ -587,7 +589,7 @@ extern "C" int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, co
                                  int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                                  int64_t topk, int64_t block_size, const int64_t* strides, float sm_scale, int dtype,
                                  void* workspace, size_t workspace_bytes, int32_t* out_segment_offsets, int32_t* out_queries,
-                                 void* stream) {
+                                 int phases, void* stream) {
   if (!q || !k || !v || !o || !dout || !lse || !topk_idx || !cu_seqlens || !dq || !dk || !dv || !strides || !workspace) return NSA_ERR_BAD_ARG;
   if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
   if ((out_segment_offsets == nullptr) != (out_queries == nullptr)) return NSA_ERR_BAD_ARG;
@@ -605,7 +607,7 @@ extern "C" int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, co
   a.ish = strides[10]; a.isn = strides[11]; a.isk = strides[12];
   a.dqsn = strides[13]; a.dqsh = strides[14]; a.dksn = strides[15]; a.dksh = strides[16]; a.dvsn = strides[17]; a.dvsh = strides[18];
   a.sm_scale = sm_scale; a.ws = (char*)workspace; a.stream = (hipStream_t)stream;
-  a.out_seg_off = out_segment_offsets; a.out_queries = out_queries;
+  a.out_seg_off = out_segment_offsets; a.out_queries = out_queries; a.phases = phases;
   if (dtype == NSA_BF16) return bwd_d<__bf16>(a);
   if (dtype == NSA_FP16) return bwd_d<_Float16>(a);
   return NSA_ERR_UNSUPPORTED;

@@ -127,32 +127,35 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
 }
 
 template <typename T, int D, int BS>
-static int launch_fwd(const TopkFwdParams& p, const void* v, long long vsn, long long vsh, hipStream_t stream) {
-  launch_block_transpose<T, D>((const T*)v, (T*)p.vt, p.cu, p.batch, vsn, vsh, p.n_slots, p.Hkv, stream);
-  long long n_wg = (p.n_items + 3) / 4;
-  n_wg = (n_wg + 7) / 8 * 8;
-  topk_fwd_kernel<T, D, BS><<<dim3((unsigned)n_wg), 256, 0, stream>>>(p);
+static int launch_fwd(const TopkFwdParams& p, const void* v, long long vsn, long long vsh, int phases, hipStream_t stream) {
+  if (phases & NSA_FWD_PHASE_TRANSPOSE)
+    launch_block_transpose<T, D>((const T*)v, (T*)p.vt, p.cu, p.batch, vsn, vsh, p.n_slots, p.Hkv, stream);
+  if (phases & NSA_FWD_PHASE_ATTEND) {
+    long long n_wg = (p.n_items + 3) / 4;
+    n_wg = (n_wg + 7) / 8 * 8;
+    topk_fwd_kernel<T, D, BS><<<dim3((unsigned)n_wg), 256, 0, stream>>>(p);
+  }
   return nsa_check_launch();
 }
 
 template <typename T, int D>
-static int dispatch_bs(int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, hipStream_t s) {
+static int dispatch_bs(int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, int ph, hipStream_t s) {
   switch (bs) {
-    case 32: return launch_fwd<T, D, 32>(p, v, vsn, vsh, s);
-    case 64: return launch_fwd<T, D, 64>(p, v, vsn, vsh, s);
-    case 128: return launch_fwd<T, D, 128>(p, v, vsn, vsh, s);
-    case 256: return launch_fwd<T, D, 256>(p, v, vsn, vsh, s);
+    case 32: return launch_fwd<T, D, 32>(p, v, vsn, vsh, ph, s);
+    case 64: return launch_fwd<T, D, 64>(p, v, vsn, vsh, ph, s);
+    case 128: return launch_fwd<T, D, 128>(p, v, vsn, vsh, ph, s);
+    case 256: return launch_fwd<T, D, 256>(p, v, vsn, vsh, ph, s);
   }
   return NSA_ERR_UNSUPPORTED;
 }
 
 template <typename T>
-static int dispatch_d(int d, int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, hipStream_t s) {
+static int dispatch_d(int d, int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, int ph, hipStream_t s) {
   switch (d) {
-    case 32: return dispatch_bs<T, 32>(bs, p, v, vsn, vsh, s);
-    case 64: return dispatch_bs<T, 64>(bs, p, v, vsn, vsh, s);
-    case 96: return dispatch_bs<T, 96>(bs, p, v, vsn, vsh, s);
-    case 128: return dispatch_bs<T, 128>(bs, p, v, vsn, vsh, s);
+    case 32: return dispatch_bs<T, 32>(bs, p, v, vsn, vsh, ph, s);
+    case 64: return dispatch_bs<T, 64>(bs, p, v, vsn, vsh, ph, s);
+    case 96: return dispatch_bs<T, 96>(bs, p, v, vsn, vsh, ph, s);
+    case 128: return dispatch_bs<T, 128>(bs, p, v, vsn, vsh, ph, s);
   }
   return NSA_ERR_UNSUPPORTED;
 }
@@ -167,7 +170,7 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
                                  int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
                                  int64_t v_stride_n, int64_t v_stride_h, int64_t idx_stride_h, int64_t idx_stride_n,
                                  int64_t idx_stride_k, int64_t o_stride_n, int64_t o_stride_h, float sm_scale, int dtype,
-                                 void* workspace, size_t workspace_bytes, void* stream) {
+                                 void* workspace, size_t workspace_bytes, int phases, void* stream) {
   if (!q || !k || !v || !topk_idx || !o || !lse || !cu_seqlens || !workspace) return NSA_ERR_BAD_ARG;
   if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
   if (total_len >= (1ll << 31)) return NSA_ERR_BAD_ARG;
@@ -185,8 +188,8 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   p.ish = idx_stride_h; p.isn = idx_stride_n; p.isk = idx_stride_k; p.osn = o_stride_n; p.osh = o_stride_h;
   p.qk_scale = sm_scale * NSA_LOG2E;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, s);
-  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, s);
+  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, phases, s);
+  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, phases, s);
   return NSA_ERR_UNSUPPORTED;
 }
 

@@ -19,10 +19,10 @@ P, I, F, Z = c_void_p, c_int64, c_float, c_size_t
 _SIGNATURES = {
     "nsa_version": (c_int, []),
     "nsa_topk_attn_fwd_workspace_bytes": (Z, [I, I, I, I]),
-    "nsa_topk_attn_fwd": (c_int, [P] * 7 + [I] * 7 + [I] * 11 + [F, c_int, P, Z, P]),
+    "nsa_topk_attn_fwd": (c_int, [P] * 7 + [I] * 7 + [I] * 11 + [F, c_int, P, Z, c_int, P]),
     "nsa_topk_attn_bwd_workspace_bytes": (Z, [I] * 7),
     "nsa_topk_reverse_index_segments": (I, [I] * 4),
-    "nsa_topk_attn_bwd": (c_int, [P] * 11 + [I] * 7 + [P, F, c_int, P, Z, P, P, P]),
+    "nsa_topk_attn_bwd": (c_int, [P] * 11 + [I] * 7 + [P, F, c_int, P, Z, P, P, c_int, P]),
 }
 
 

@@ -12,8 +12,11 @@ def _last_dim_contiguous(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
-def _topk_sparse_attention_fwd(q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale):
-    """Returns (o [T,Hq,D], lse fp32 [Hq,T] in base-2 units); mirrors _topk_sparse_attention_fwd (:828-909)."""
+def _topk_sparse_attention_fwd(q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale,
+                               workspace=None, phases=3, out=None):
+    """Returns (o [T,Hq,D], lse fp32 [Hq,T] in base-2 units); mirrors _topk_sparse_attention_fwd (:828-909).
+
+    workspace / phases / out let a profiler re-run one pass on buffers a previous call filled."""
     assert k.dtype == q.dtype and v.dtype == q.dtype
     assert cu_seqlens_q.dtype == torch.int32 and cu_seqlens_k.dtype == torch.int32
     assert block_size in {32, 64, 128, 256}
@@ -26,23 +29,28 @@ def _topk_sparse_attention_fwd(q, k, v, topk_idx, block_size, cu_seqlens_q, cu_s
     assert topk_idx.shape[0] == num_k_heads and topk_idx.shape[1] == q_len
     assert num_k_heads == num_v_heads and num_q_heads % num_k_heads == 0
     q, k, v = map(_last_dim_contiguous, (q, k, v))
-    o = torch.empty((q_len, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
-    lse = torch.empty((num_q_heads, q_len), dtype=torch.float32, device=q.device)
+    if out is None:
+        o = torch.empty((q_len, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+        lse = torch.empty((num_q_heads, q_len), dtype=torch.float32, device=q.device)
+    else:
+        o, lse = out
     lib = _lib.load()
-    ws = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(q_len, batch, num_k_heads, head_dim), q.device)
+    ws = workspace
+    if ws is None:
+        ws = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(q_len, batch, num_k_heads, head_dim), q.device)
     rc = lib.nsa_topk_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), topk_idx.data_ptr(), o.data_ptr(), lse.data_ptr(),
         cu_seqlens_q.data_ptr(), q_len, batch, num_q_heads, num_k_heads, head_dim, topk, block_size,
         q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
         topk_idx.stride(0), topk_idx.stride(1), topk_idx.stride(2), o.stride(0), o.stride(1),
-        sm_scale, _lib.dtype_code(q), ws.data_ptr(), ws.numel(), _lib.stream_ptr(q),
+        sm_scale, _lib.dtype_code(q), ws.data_ptr(), ws.numel(), phases, _lib.stream_ptr(q),
     )
     _lib.check(rc, "nsa_topk_attn_fwd")
     return o, lse
 
 
 def _topk_sparse_attention_bwd(o, do, lse, q, k, v, topk_idx, block_size, cu_seqlens_q, cu_seqlens_k,
-                               max_seqlen_q, max_seqlen_k, sm_scale, return_reverse_index=False):
+                               max_seqlen_q, max_seqlen_k, sm_scale, return_reverse_index=False, workspace=None, phases=7, out=None):
     """Returns (dq, dk, dv); mirrors _topk_sparse_attention_bwd (:912-1109)."""
     assert block_size in {32, 64, 128, 256}
     q_len, num_q_heads, head_dim = q.shape
@@ -50,12 +58,17 @@ def _topk_sparse_attention_bwd(o, do, lse, q, k, v, topk_idx, block_size, cu_seq
     batch = cu_seqlens_q.shape[0] - 1
     topk = topk_idx.shape[-1]
     q, k, v, o, do = map(_last_dim_contiguous, (q, k, v, o, do))
-    dq = torch.empty((q_len, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
-    dk = torch.empty((q_len, num_k_heads, head_dim), dtype=q.dtype, device=q.device)
-    dv = torch.empty((q_len, num_k_heads, head_dim), dtype=q.dtype, device=q.device)
+    if out is None:
+        dq = torch.empty((q_len, num_q_heads, head_dim), dtype=q.dtype, device=q.device)
+        dk = torch.empty((q_len, num_k_heads, head_dim), dtype=q.dtype, device=q.device)
+        dv = torch.empty((q_len, num_k_heads, head_dim), dtype=q.dtype, device=q.device)
+    else:
+        dq, dk, dv = out
     lib = _lib.load()
-    ws = _lib.workspace(
-        lib.nsa_topk_attn_bwd_workspace_bytes(q_len, batch, num_q_heads, num_k_heads, head_dim, topk, block_size), q.device)
+    ws = workspace
+    if ws is None:
+        ws = _lib.workspace(
+            lib.nsa_topk_attn_bwd_workspace_bytes(q_len, batch, num_q_heads, num_k_heads, head_dim, topk, block_size), q.device)
     strides = _lib.host_i64(
         [q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), o.stride(0), o.stride(1),
          do.stride(0), do.stride(1), topk_idx.stride(0), topk_idx.stride(1), topk_idx.stride(2),
@@ -70,7 +83,7 @@ def _topk_sparse_attention_bwd(o, do, lse, q, k, v, topk_idx, block_size, cu_seq
         cu_seqlens_q.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), q_len, batch, num_q_heads, num_k_heads,
         head_dim, topk, block_size, strides, sm_scale, _lib.dtype_code(q), ws.data_ptr(), ws.numel(),
         seg_off.data_ptr() if return_reverse_index else None, queries.data_ptr() if return_reverse_index else None,
-        _lib.stream_ptr(q),
+        phases, _lib.stream_ptr(q),
     )
     _lib.check(rc, "nsa_topk_attn_bwd")
     if return_reverse_index:
