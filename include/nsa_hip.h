@@ -84,6 +84,27 @@ int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, const void* o
                       size_t workspace_bytes, int32_t* out_segment_offsets, int32_t* out_queries, int phases,
                       void* stream);
 
+/* ---- weightedpool_compress / avgpool_compress ---------------------------------------------
+ * Forward: replaces sliding_pool_fwd_kernel (native_sparse_attention/ops/triton/weighted_pool.py:24-85,
+ * launched at :218-236).  x [total_x,H,D]; w [H,kernel_size] in the dtype of x, or NULL for the
+ * average; y [total_y,H,D]; y_cu_seqlens int32 [batch+1] as computed by get_compressed_seqlens
+ * (ops/triton/utils.py:25-37).  The positional-embedding bias stays in the caller as in the reference.
+ */
+int nsa_pool_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
+                 int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim, int64_t kernel_size,
+                 int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h, int64_t y_stride_n, int64_t y_stride_h,
+                 int64_t w_stride_h, int dtype, void* stream);
+/* Backward: replaces sliding_pool_dxdw_kernel (:89-179, launched at :262-292) and the dw.sum(1)
+ * that follows (:297).  dx is a gather over the windows covering each token (no atomics);
+ * dw (NULL iff w is NULL) is reduced over fp32 per-tile partials held in the workspace.
+ */
+size_t nsa_pool_bwd_workspace_bytes(int64_t total_y, int64_t num_heads, int64_t kernel_size);
+int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, const int32_t* cu_seqlens,
+                 const int32_t* y_cu_seqlens, int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads,
+                 int64_t head_dim, int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
+                 int64_t dy_stride_n, int64_t dy_stride_h, int64_t dx_stride_n, int64_t dx_stride_h, int64_t w_stride_h,
+                 int64_t dw_stride_h, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

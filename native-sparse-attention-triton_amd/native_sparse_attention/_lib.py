@@ -23,6 +23,9 @@ _SIGNATURES = {
     "nsa_topk_attn_bwd_workspace_bytes": (Z, [I] * 7),
     "nsa_topk_reverse_index_segments": (I, [I] * 4),
     "nsa_topk_attn_bwd": (c_int, [P] * 11 + [I] * 7 + [P, F, c_int, P, Z, P, P, c_int, P]),
+    "nsa_pool_fwd": (c_int, [P] * 5 + [I] * 12 + [c_int, P]),
+    "nsa_pool_bwd_workspace_bytes": (Z, [I] * 3),
+    "nsa_pool_bwd": (c_int, [P] * 7 + [I] * 15 + [c_int, P, Z, P]),
 }
 
 

@@ -1,0 +1,21 @@
+"""Host-side helpers shared by the operators."""
+import torch
+
+
+def get_compressed_seqlens(cu_seqlens: torch.Tensor, kernel_size: int, kernel_stride: int):
+    """Per-sequence lengths after sliding-window compression and their cumulative sum.
+
+    y_len = floor((L - kernel_size) / kernel_stride) + 1, or 0 when L < kernel_size; both results are
+    int32 on the device of ``cu_seqlens`` (same contract as the reference's
+    native_sparse_attention/ops/triton/utils.py:25-37).
+    """
+    seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
+    y_seqlens = torch.div(seqlens - kernel_size, kernel_stride, rounding_mode="floor").to(torch.int32) + 1
+    y_seqlens = torch.where(seqlens < kernel_size, torch.zeros_like(y_seqlens), y_seqlens)
+    y_cu_seqlens = torch.zeros(y_seqlens.shape[0] + 1, dtype=torch.int32, device=cu_seqlens.device)
+    y_cu_seqlens[1:] = torch.cumsum(y_seqlens, dim=0)
+    return y_seqlens, y_cu_seqlens
+
+
+def last_dim_contiguous(t: torch.Tensor) -> torch.Tensor:
+    return t if t.stride(-1) == 1 else t.contiguous()
