@@ -105,6 +105,41 @@ int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* dx, void* d
                  int64_t dy_stride_n, int64_t dy_stride_h, int64_t dx_stride_n, int64_t dx_stride_h, int64_t w_stride_h,
                  int64_t dw_stride_h, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- decode (one query per sequence over KV-cache slabs [B, slab_len, Hkv, D]) ---------------
+ * strides: HOST int64 array: q(b,h) k(b,n,h) v(b,n,h) o(b,h) [+ idx(h,b,k) for the entry points
+ * that read or write topk ids] = 10 or 13 values.  q/k/v strides must be multiples of 8.
+ *
+ * nsa_dense_decode replaces decode_kernel (native_sparse_attention/ops/triton/flash_attention_decode.py:23-139,
+ * launched at :186-216): attention over the first seqlens[b] rows of the slab.
+ */
+size_t nsa_dense_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len);
+int nsa_dense_decode(const void* q, const void* k, const void* v, const int32_t* seqlens, void* o, int64_t batch,
+                     int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len, const int64_t* strides,
+                     float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+/* nsa_topk_decode replaces forward_kernel (native_sparse_attention/ops/triton/topk_sparse_attention_decode.py:23-148,
+ * launched at :199-236): topk_idx int32 [Hkv,B,topk]; ids < 0 or beyond block (seqlens[b]-1)/block_size
+ * are skipped; keys >= seqlens[b] are masked.
+ */
+size_t nsa_topk_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t topk,
+                                       int64_t block_size);
+int nsa_topk_decode(const void* q, const void* k, const void* v, const int32_t* topk_idx, const int32_t* seqlens, void* o,
+                    int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len, int64_t topk,
+                    int64_t block_size, const int64_t* strides, float sm_scale, int dtype, void* workspace,
+                    size_t workspace_bytes, void* stream);
+/* nsa_cmp_decode replaces the torch-op chain of compressed_attention_decode
+ * (native_sparse_attention/ops/torch/compressed_attention_decode.py:65-153, with transform_score :21-62):
+ * attention over the first compress_seqlens[b] rows of the compressed slab, then (if out_topk_idx is
+ * not NULL) block scores and the k_out best block ids per (kv head, sequence), ascending, ids beyond
+ * block (seqlens[b]-1)/block_size replaced by -1.  max_seqlen = max(seqlens) (host value, fixes the
+ * number of blocks); k_out <= min(64, ceil(max_seqlen/block_size)).
+ */
+size_t nsa_cmp_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len);
+int nsa_cmp_decode(const void* q, const void* k, const void* v, const int32_t* seqlens, const int32_t* compress_seqlens, void* o,
+                   int32_t* out_topk_idx, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                   int64_t slab_len, int64_t kernel_size, int64_t kernel_stride, int64_t block_size, int64_t k_out,
+                   int64_t max_seqlen, int64_t init_blocks, int64_t local_blocks, const int64_t* strides, float sm_scale,
+                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,399 @@
+// Single-query (decode) attention over KV-cache slabs [B, max_len, Hkv, D]:
+//   dense      - the first seqlens[b] rows (sliding-window ring, plain KV cache)
+//   top-k      - the 64-token-aligned blocks named by topk_idx[h, b, :]
+//   compressed - dense over the compressed slab, then per-key probabilities summed over the GQA
+//                group -> overlap-weighted block scores -> forced init/local blocks -> top-k ids
+// All three share one split-K kernel: a workgroup takes 64 keys of one (sequence, kv-head), each
+// wave 16 of them, with the (up to 16) query heads of the group as MFMA columns; partial
+// (max, sum, O) triples go to the workspace and a second kernel merges them.  The work is a few
+// MiB per step, so the aim is few launches and coalesced 16-byte accesses, not MFMA rate.
+#include "nsa_common.h"
+
+struct DecodeParams {
+  const void* q; const void* k; const void* v; const int32_t* lens; const int32_t* idx;
+  float* pm; float* pl; float* po;
+  int B, Hkv, G, GT, n_chunks, topk, bs, slab_len;
+  long long qsb, qsh, ksb, ksn, ksh, vsb, vsn, vsh, ish, isb, isk;
+  float qk_scale;
+};
+
+// MODE 0: dense prefix, MODE 1: top-k blocks
+template <typename T, int D, int MODE>
+__global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8;
+  __shared__ __attribute__((aligned(16))) T v_s[4][16][LD];
+  __shared__ float m_s[4][16], l_s[4][16];
+  __shared__ float o_s[16][D + 1];
+  const int chunk = blockIdx.x, h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const int len = min(p.lens[b], p.slab_len);  // never read past the slab
+  int k0, kend;  // keys [k0, kend) of this chunk are visible
+  if (MODE == 0) {
+    k0 = chunk * 64;
+    kend = min(len, k0 + 64);
+  } else {
+    const int cpb = p.bs >= 64 ? p.bs / 64 : 1;
+    const int e = chunk / cpb, sub = chunk % cpb;
+    const int blk = p.idx[(long long)h * p.ish + (long long)b * p.isb + (long long)e * p.isk];
+    const bool ok = blk >= 0 && len > 0 && blk <= (len - 1) / p.bs;
+    k0 = ok ? blk * p.bs + 64 * sub : 0;
+    kend = ok ? min(len, min(k0 + 64, (blk + 1) * p.bs)) : 0;
+  }
+  const long long slot = (((long long)b * p.Hkv + h) * p.GT + gt) * p.n_chunks + chunk;
+  float* pm = p.pm + slot * 16;
+  float* pl = p.pl + slot * 16;
+  float* po = p.po + slot * 16 * D;
+  if (kend <= k0) {  // nothing visible: neutral partial
+    if (tid < 16) { pm[tid] = -INFINITY; pl[tid] = 0.f; }
+    for (int i = tid; i < 16 * D; i += 256) po[i] = 0.f;
+    return;
+  }
+  const int hq = gt * 16 + li;
+  const bool has_head = hq < p.G;
+  const T* qp = (const T*)p.q + (long long)b * p.qsb + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
+  v8 qf[NK];
+#pragma unroll
+  for (int kk = 0; kk < NK; kk++) qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+  // this wave's 16 keys
+  const int kw = k0 + 16 * wave;
+  {
+    const int key = kw + li;
+    const int row = key < kend ? key : k0;
+    const T* kp = (const T*)p.k + (long long)b * p.ksb + (long long)row * p.ksn + (long long)h * p.ksh + 8 * lg;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    if (kw < kend) {
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) s = E::mfma16(ld16<v8>(kp + 32 * kk), qf[kk], s);
+    }
+    // stage V rows (zeros for invisible keys: slab rows past the length may hold anything)
+    constexpr int PIECES = 16 * (D / 8);
+    for (int i = lane; i < PIECES; i += 64) {
+      const int r = i / (D / 8), c = (i % (D / 8)) * 8;
+      uint4 val = {0u, 0u, 0u, 0u};
+      if (kw + r < kend) val = *reinterpret_cast<const uint4*>((const T*)p.v + (long long)b * p.vsb + (long long)(kw + r) * p.vsn + (long long)h * p.vsh + c);
+      *reinterpret_cast<uint4*>(&v_s[wave][r][c]) = val;
+    }
+    float mw = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float x = (kw + 4 * lg + r) < kend ? s[r] * p.qk_scale : -INFINITY;
+      s[r] = x;
+      mw = fmaxf(mw, x);
+    }
+    mw = fmaxf(mw, __shfl_xor(mw, 16));
+    mw = fmaxf(mw, __shfl_xor(mw, 32));
+    float lw = 0.f;
+    v8 pf = zero16<v8>();
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float x = mw == -INFINITY ? 0.f : fast_exp2(s[r] - mw);
+      lw += x;
+      pf[r] = (T)x;
+    }
+    lw += __shfl_xor(lw, 16);
+    lw += __shfl_xor(lw, 32);
+    if (lg == 0) { m_s[wave][li] = mw; l_s[wave][li] = lw; }
+    __syncthreads();  // v_s staged, m_s/l_s visible
+    float m = fmaxf(fmaxf(m_s[0][li], m_s[1][li]), fmaxf(m_s[2][li], m_s[3][li]));
+    const float sc = mw == -INFINITY ? 0.f : fast_exp2(mw - m);
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    f32x4 acc[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) {
+      const T* va = &v_s[wave][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+      s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(va));
+      s16x8 a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
+      f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      acc[dt] = E::mfma16(__builtin_bit_cast(v8, a8), pf, z);
+    }
+    // o_s[head][d] = sum over waves of sc * acc, one wave at a time
+    for (int w = 0; w < 4; w++) {
+      if (wave == w) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            float* dst = &o_s[li][16 * dt + 4 * lg + r];
+            *dst = (w == 0 ? 0.f : *dst) + sc * acc[dt][r];
+          }
+      }
+      __syncthreads();
+    }
+    if (tid < 16) {
+      float mm = fmaxf(fmaxf(m_s[0][tid], m_s[1][tid]), fmaxf(m_s[2][tid], m_s[3][tid]));
+      float ll = 0.f;
+      for (int w = 0; w < 4; w++) ll += m_s[w][tid] == -INFINITY ? 0.f : l_s[w][tid] * fast_exp2(m_s[w][tid] - mm);
+      pm[tid] = mm;
+      pl[tid] = ll;
+    }
+    for (int i = tid; i < 16 * D; i += 256) po[i] = o_s[i / D][i % D];
+  }
+}
+
+// merge the chunk partials of one (sequence, query head); optionally keep the base-2 LSE
+template <typename T, int D>
+__global__ void decode_merge_kernel(DecodeParams p, T* __restrict__ o, long long osb, long long osh, float* __restrict__ lse) {
+  const int hq_all = blockIdx.x, b = blockIdx.y;
+  const int h = hq_all / p.G, hq = hq_all % p.G, gt = hq / 16, col = hq % 16;
+  const long long base = (((long long)b * p.Hkv + h) * p.GT + gt) * p.n_chunks;
+  float m = -INFINITY;
+  for (int c = 0; c < p.n_chunks; c++) m = fmaxf(m, p.pm[(base + c) * 16 + col]);
+  float l = 0.f;
+  for (int c = 0; c < p.n_chunks; c++) {
+    const float mc = p.pm[(base + c) * 16 + col];
+    if (mc != -INFINITY) l += p.pl[(base + c) * 16 + col] * fast_exp2(mc - m);
+  }
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f;
+    for (int c = 0; c < p.n_chunks; c++) {
+      const float mc = p.pm[(base + c) * 16 + col];
+      if (mc != -INFINITY) acc += p.po[((base + c) * 16 + col) * D + d] * fast_exp2(mc - m);
+    }
+    o[(long long)b * osb + (long long)hq_all * osh + d] = (T)(l > 0.f ? acc / l : 0.f);
+  }
+  if (lse && threadIdx.x == 0) lse[(long long)b * p.Hkv * p.G + hq_all] = l > 0.f ? m + fast_log2(l) : INFINITY;
+}
+
+// ------------------------------------------------------------------------------------------
+// compressed decode: probabilities -> block scores -> top-k ids
+struct ScoreParams {
+  const void* q; const void* k; const float* lse; const int32_t* seqlens; const int32_t* clens; float* score; int32_t* out_idx;
+  int B, Hkv, G, GT, slab_len, ks, st, bs, init_blocks, local_blocks, k_out, max_blocks, full_blocks;
+  long long qsb, qsh, ksb, ksn, ksh, osh, osb, osk;
+  float qk_scale;
+};
+
+static constexpr int MAX_SCORE_BLOCKS = 8192;
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void decode_score_select_kernel(ScoreParams p) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  constexpr int NK = D / 32;
+  __shared__ float bscore[MAX_SCORE_BLOCKS];
+  __shared__ float red_v[256];
+  __shared__ int red_i[256];
+  __shared__ int picked[64];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const int lc = min(p.clens[b], p.slab_len);
+  float* score = p.score + ((long long)b * p.Hkv + h) * p.slab_len;
+  // phase A: score[c] = sum over the group's heads of exp2(s*scale - lse)
+  for (int sub = wave; sub * 16 < lc; sub += 4) {
+    f32x4 tot = {0.f, 0.f, 0.f, 0.f};
+    const int key = sub * 16 + li;
+    const int row = key < lc ? key : 0;
+    const T* kp = (const T*)p.k + (long long)b * p.ksb + (long long)row * p.ksn + (long long)h * p.ksh + 8 * lg;
+    for (int gt = 0; gt < p.GT; gt++) {
+      const int hq = gt * 16 + li;
+      const bool has_head = hq < p.G;
+      const T* qp = (const T*)p.q + (long long)b * p.qsb + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
+      const float l2 = has_head ? p.lse[(long long)b * p.Hkv * p.G + h * p.G + hq] : INFINITY;
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) s = E::mfma16(ld16<v8>(kp + 32 * kk), has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>(), s);
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        float x = (sub * 16 + 4 * lg + r) < lc ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
+        x += __shfl_xor(x, 1); x += __shfl_xor(x, 2); x += __shfl_xor(x, 4); x += __shfl_xor(x, 8);
+        tot[r] += x;
+      }
+    }
+    if (li == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) if (sub * 16 + 4 * lg + r < lc) score[sub * 16 + 4 * lg + r] = tot[r];
+    }
+  }
+  __syncthreads();
+  // phase B: block scores
+  const int a = p.ks / p.st, rr = p.bs / p.st, pad = a - 1;
+  const int qb = (p.seqlens[b] - 1) / p.bs;
+  for (int blk = tid; blk < p.max_blocks; blk += 256) {
+    float v = 0.f;
+    if (blk < p.full_blocks) {
+      for (int o = 0; o < a + rr - 1; o++) {
+        const int c = blk * rr + o - pad;
+        const int w = min(min(o, a + rr - 2 - o), min(a - 1, rr - 1)) + 1;
+        if (c >= 0 && c < lc) v += (float)w * score[c];
+      }
+    }
+    if (v != v) v = 0.f;
+    if (blk < p.init_blocks || (blk <= qb && blk > qb - p.local_blocks)) v = INFINITY;
+    bscore[blk] = v;
+  }
+  __syncthreads();
+  // phase C: k_out rounds of (largest value, smallest index)
+  for (int round = 0; round < p.k_out; round++) {
+    float bv = -1.f;
+    int bi = 0x7fffffff;
+    for (int blk = tid; blk < p.max_blocks; blk += 256) {
+      const float v = bscore[blk];
+      if (v > bv) { bv = v; bi = blk; }
+    }
+    red_v[tid] = bv; red_i[tid] = bi;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+      if (tid < s) {
+        const float ov = red_v[tid + s]; const int oi = red_i[tid + s];
+        if (ov > red_v[tid] || (ov == red_v[tid] && oi < red_i[tid])) { red_v[tid] = ov; red_i[tid] = oi; }
+      }
+      __syncthreads();
+    }
+    if (tid == 0) { picked[round] = red_i[0]; bscore[red_i[0]] = -2.f; }
+    __syncthreads();
+  }
+  // ascending order, ids beyond the query's block become -1 at the tail
+  if (tid == 0) {
+    int32_t* out = p.out_idx + (long long)h * p.osh + (long long)b * p.osb;
+    for (int i = 1; i < p.k_out; i++) {  // insertion sort of <= 64 ids
+      int x = picked[i], j = i - 1;
+      while (j >= 0 && picked[j] > x) { picked[j + 1] = picked[j]; j--; }
+      picked[j + 1] = x;
+    }
+    for (int i = 0; i < p.k_out; i++) out[(long long)i * p.osk] = picked[i] > qb ? -1 : picked[i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+static inline int chunks_for(int mode, int64_t slab_len, int64_t topk, int64_t bs) {
+  return mode == 0 ? (int)((slab_len + 63) / 64) : (int)(topk * (bs >= 64 ? bs / 64 : 1));
+}
+
+static size_t decode_partial_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int n_chunks) {
+  const int64_t GT = (Hq / Hkv + 15) / 16;
+  return (size_t)(B * Hkv * GT * n_chunks) * 16 * (size_t)(D + 2) * 4;
+}
+
+template <typename T, int D>
+static int run_decode(int mode, DecodeParams& p, void* o, long long osb, long long osh, float* lse, char* ws, hipStream_t s) {
+  const size_t n = (size_t)p.B * p.Hkv * p.GT * p.n_chunks * 16;
+  p.pm = (float*)ws; p.pl = p.pm + n; p.po = p.pl + n;
+  dim3 grid((unsigned)p.n_chunks, (unsigned)(p.Hkv * p.GT), (unsigned)p.B);
+  if (mode == 0) decode_partial_kernel<T, D, 0><<<grid, 256, 0, s>>>(p);
+  else decode_partial_kernel<T, D, 1><<<grid, 256, 0, s>>>(p);
+  decode_merge_kernel<T, D><<<dim3((unsigned)(p.Hkv * p.G), (unsigned)p.B), D <= 64 ? 64 : 128, 0, s>>>(p, (T*)o, osb, osh, lse);
+  return nsa_check_launch();
+}
+
+#define DECODE_DISPATCH(CALL)                                                   \
+  switch (head_dim) {                                                           \
+    case 32: return dtype == NSA_BF16 ? CALL(__bf16, 32) : CALL(_Float16, 32);  \
+    case 64: return dtype == NSA_BF16 ? CALL(__bf16, 64) : CALL(_Float16, 64);  \
+    case 96: return dtype == NSA_BF16 ? CALL(__bf16, 96) : CALL(_Float16, 96);  \
+    case 128: return dtype == NSA_BF16 ? CALL(__bf16, 128) : CALL(_Float16, 128); \
+  }                                                                             \
+  return NSA_ERR_UNSUPPORTED;
+
+static int fill_decode(DecodeParams& p, const void* q, const void* k, const void* v, const int32_t* lens, int64_t B, int64_t Hq,
+                       int64_t Hkv, int64_t slab_len, const int64_t* st, float sm_scale) {
+  if (!q || !k || !v || !lens || !st || B <= 0 || Hkv <= 0 || Hq % Hkv != 0 || slab_len <= 0) return NSA_ERR_BAD_ARG;
+  for (int i = 0; i < 8; i++) if (st[i] % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 != 0) return NSA_ERR_UNSUPPORTED;
+  p.q = q; p.k = k; p.v = v; p.lens = lens; p.idx = nullptr; p.B = (int)B; p.Hkv = (int)Hkv; p.G = (int)(Hq / Hkv);
+  p.GT = (p.G + 15) / 16; p.slab_len = (int)slab_len; p.topk = 0; p.bs = 64;
+  p.qsb = st[0]; p.qsh = st[1]; p.ksb = st[2]; p.ksn = st[3]; p.ksh = st[4]; p.vsb = st[5]; p.vsn = st[6]; p.vsh = st[7];
+  p.ish = p.isb = p.isk = 0; p.qk_scale = sm_scale * NSA_LOG2E;
+  return NSA_OK;
+}
+
+extern "C" size_t nsa_dense_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len) {
+  return decode_partial_bytes(batch, num_q_heads, num_kv_heads, head_dim, chunks_for(0, slab_len, 0, 64));
+}
+
+extern "C" int nsa_dense_decode(const void* q, const void* k, const void* v, const int32_t* seqlens, void* o, int64_t batch,
+                                int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len,
+                                const int64_t* strides, float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  DecodeParams p;
+  int rc = fill_decode(p, q, k, v, seqlens, batch, num_q_heads, num_kv_heads, slab_len, strides, sm_scale);
+  if (rc != NSA_OK) return rc;
+  if (!o || !workspace) return NSA_ERR_BAD_ARG;
+  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_dense_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, slab_len)) return NSA_ERR_WORKSPACE;
+  p.n_chunks = chunks_for(0, slab_len, 0, 64);
+  const long long osb = strides[8], osh = strides[9];
+  hipStream_t s = (hipStream_t)stream;
+#define CALL(T, D) run_decode<T, D>(0, p, o, osb, osh, nullptr, (char*)workspace, s)
+  DECODE_DISPATCH(CALL)
+#undef CALL
+}
+
+extern "C" size_t nsa_topk_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                                  int64_t topk, int64_t block_size) {
+  return decode_partial_bytes(batch, num_q_heads, num_kv_heads, head_dim, chunks_for(1, 0, topk, block_size));
+}
+
+extern "C" int nsa_topk_decode(const void* q, const void* k, const void* v, const int32_t* topk_idx, const int32_t* seqlens, void* o,
+                               int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len,
+                               int64_t topk, int64_t block_size, const int64_t* strides, float sm_scale, int dtype,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  DecodeParams p;
+  int rc = fill_decode(p, q, k, v, seqlens, batch, num_q_heads, num_kv_heads, slab_len, strides, sm_scale);
+  if (rc != NSA_OK) return rc;
+  if (!o || !workspace || !topk_idx || topk <= 0) return NSA_ERR_BAD_ARG;
+  if (block_size != 32 && block_size != 64 && block_size != 128 && block_size != 256) return NSA_ERR_UNSUPPORTED;
+  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_topk_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, topk, block_size)) return NSA_ERR_WORKSPACE;
+  p.idx = topk_idx; p.topk = (int)topk; p.bs = (int)block_size;
+  p.ish = strides[10]; p.isb = strides[11]; p.isk = strides[12];
+  p.n_chunks = chunks_for(1, 0, topk, block_size);
+  const long long osb = strides[8], osh = strides[9];
+  hipStream_t s = (hipStream_t)stream;
+#define CALL(T, D) run_decode<T, D>(1, p, o, osb, osh, nullptr, (char*)workspace, s)
+  DECODE_DISPATCH(CALL)
+#undef CALL
+}
+
+static size_t cmp_decode_partial(int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t slab_len) {
+  return (decode_partial_bytes(B, Hq, Hkv, D, chunks_for(0, slab_len, 0, 64)) + 255) & ~(size_t)255;
+}
+
+extern "C" size_t nsa_cmp_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len) {
+  return cmp_decode_partial(batch, num_q_heads, num_kv_heads, head_dim, slab_len) + (size_t)batch * num_q_heads * 4 + 256 +
+         (size_t)batch * num_kv_heads * slab_len * 4;
+}
+
+template <typename T, int D>
+static int run_cmp_decode(DecodeParams& p, ScoreParams& sp, void* o, long long osb, long long osh, char* ws, size_t part_bytes, hipStream_t s) {
+  float* lse = (float*)(ws + part_bytes);
+  float* score = (float*)(ws + part_bytes + (((size_t)p.B * p.Hkv * p.G * 4 + 255) & ~(size_t)255));
+  int rc = run_decode<T, D>(0, p, o, osb, osh, lse, ws, s);
+  if (rc != NSA_OK) return rc;
+  if (sp.out_idx) {
+    sp.lse = lse; sp.score = score;
+    decode_score_select_kernel<T, D><<<dim3((unsigned)p.Hkv, (unsigned)p.B), 256, 0, s>>>(sp);
+  }
+  return nsa_check_launch();
+}
+
+extern "C" int nsa_cmp_decode(const void* q, const void* k, const void* v, const int32_t* seqlens, const int32_t* compress_seqlens,
+                              void* o, int32_t* out_topk_idx, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                              int64_t head_dim, int64_t slab_len, int64_t kernel_size, int64_t kernel_stride, int64_t block_size,
+                              int64_t k_out, int64_t max_seqlen, int64_t init_blocks, int64_t local_blocks, const int64_t* strides,
+                              float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  DecodeParams p;
+  int rc = fill_decode(p, q, k, v, compress_seqlens, batch, num_q_heads, num_kv_heads, slab_len, strides, sm_scale);
+  if (rc != NSA_OK) return rc;
+  if (!o || !workspace || !seqlens) return NSA_ERR_BAD_ARG;
+  if (kernel_stride <= 0 || kernel_size % kernel_stride != 0 || block_size % kernel_size != 0) return NSA_ERR_BAD_ARG;
+  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_cmp_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, slab_len)) return NSA_ERR_WORKSPACE;
+  const int64_t max_blocks = (max_seqlen + block_size - 1) / block_size;
+  if (out_topk_idx && (k_out <= 0 || k_out > 64 || k_out > max_blocks || max_blocks > MAX_SCORE_BLOCKS)) return NSA_ERR_UNSUPPORTED;
+  p.n_chunks = chunks_for(0, slab_len, 0, 64);
+  ScoreParams sp;
+  sp.q = q; sp.k = k; sp.seqlens = seqlens; sp.clens = compress_seqlens; sp.out_idx = out_topk_idx;
+  sp.B = p.B; sp.Hkv = p.Hkv; sp.G = p.G; sp.GT = p.GT; sp.slab_len = p.slab_len; sp.ks = (int)kernel_size; sp.st = (int)kernel_stride;
+  sp.bs = (int)block_size; sp.init_blocks = (int)init_blocks; sp.local_blocks = (int)local_blocks; sp.k_out = (int)k_out;
+  sp.max_blocks = (int)max_blocks; sp.full_blocks = (int)(max_seqlen / block_size);
+  sp.qsb = p.qsb; sp.qsh = p.qsh; sp.ksb = p.ksb; sp.ksn = p.ksn; sp.ksh = p.ksh;
+  sp.osh = strides[10]; sp.osb = strides[11]; sp.osk = strides[12]; sp.qk_scale = p.qk_scale;
+  const long long osb = strides[8], osh = strides[9];
+  const size_t part = cmp_decode_partial(batch, num_q_heads, num_kv_heads, head_dim, slab_len);
+  hipStream_t s = (hipStream_t)stream;
+#define CALL(T, D) run_cmp_decode<T, D>(p, sp, o, osb, osh, (char*)workspace, part, s)
+  DECODE_DISPATCH(CALL)
+#undef CALL
+}

@@ -26,6 +26,12 @@ _SIGNATURES = {
     "nsa_pool_fwd": (c_int, [P] * 5 + [I] * 12 + [c_int, P]),
     "nsa_pool_bwd_workspace_bytes": (Z, [I] * 3),
     "nsa_pool_bwd": (c_int, [P] * 7 + [I] * 15 + [c_int, P, Z, P]),
+    "nsa_dense_decode_workspace_bytes": (Z, [I] * 5),
+    "nsa_dense_decode": (c_int, [P] * 5 + [I] * 5 + [P, F, c_int, P, Z, P]),
+    "nsa_topk_decode_workspace_bytes": (Z, [I] * 6),
+    "nsa_topk_decode": (c_int, [P] * 6 + [I] * 7 + [P, F, c_int, P, Z, P]),
+    "nsa_cmp_decode_workspace_bytes": (Z, [I] * 5),
+    "nsa_cmp_decode": (c_int, [P] * 7 + [I] * 12 + [P, F, c_int, P, Z, P]),
 }
 
 

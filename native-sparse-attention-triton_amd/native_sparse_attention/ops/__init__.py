@@ -1,9 +1,17 @@
 """Drop-in operator surface of native_sparse_attention.ops, backed by libnsa_hip.so."""
 from .weighted_pool import avgpool_compress, weightedpool_compress  # noqa: F401
 from .topk_sparse_attention import topk_sparse_attention  # noqa: F401
+from .decode import (  # noqa: F401
+    compressed_attention_decode,
+    flash_attention_decode,
+    topk_sparse_attention_decode,
+)
 
 __all__ = [
     "avgpool_compress",
     "weightedpool_compress",
     "topk_sparse_attention",
+    "flash_attention_decode",
+    "compressed_attention_decode",
+    "topk_sparse_attention_decode",
 ]
