@@ -105,6 +105,41 @@ int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* dx, void* d
                  int64_t dy_stride_n, int64_t dy_stride_h, int64_t dx_stride_n, int64_t dx_stride_h, int64_t w_stride_h,
                  int64_t dw_stride_h, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- compressed_attention --------------------------------------------------------------------
+ * Forward: replaces forward_kernel launched from _compressed_attention_fwd
+ * (native_sparse_attention/ops/triton/compressed_attention.py:538-640).  q,o [Tq,Hq,D];
+ * k,v [Tk,Hkv,D] compressed keys/values; query position i of a sequence sees its compressed key c
+ * iff c*kernel_stride + kernel_size - 1 <= i; rows that see nothing get o = 0, lse = -inf.
+ * lse fp32 [Hq,Tq] base-2.  strides (HOST int64[8]): q(n,h) k(n,h) v(n,h) o(n,h).
+ */
+int nsa_cmp_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens_q,
+                     const int32_t* cu_seqlens_k, int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads,
+                     int64_t num_kv_heads, int64_t head_dim, int64_t kernel_size, int64_t kernel_stride,
+                     const int64_t* strides, float sm_scale, int dtype, void* stream);
+/* Block selection: replaces score_kernel + _transform_score_kernel + torch.topk/sort/mask
+ * (:852-1179 and :1263-1292; the dense [Hkv,Tq,Tk] score tensor is never materialised).
+ * out_topk_idx int32 [Hkv,Tq,k_out], k_out <= ceil(max_seqlen_q/block_size): ids of the k_out
+ * best-scoring blocks per (kv head, token) in ascending order, -1 padded; init_blocks first and
+ * local_blocks last causal blocks are always selected.  strides (HOST int64[9]):
+ * q(n,h) k(n,h) 0 0 idx(h,n,k).
+ */
+int nsa_cmp_attn_select(const void* q, const void* k, const float* lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                        int32_t* out_topk_idx, int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads,
+                        int64_t num_kv_heads, int64_t head_dim, int64_t kernel_size, int64_t kernel_stride, int64_t block_size,
+                        int64_t k_out, int64_t max_seqlen_q, int64_t init_blocks, int64_t local_blocks, const int64_t* strides,
+                        float sm_scale, int dtype, void* stream);
+/* Backward: replaces backward_sum_o_do, backward_dkdv (+ the .sum(0) over bf16 per-head partials)
+ * and backward_dq launched from _compressed_attention_bwd (:643-780).
+ * strides (HOST int64[16]): q k v o dout dq dk dv, (n,h) each.
+ */
+size_t nsa_cmp_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                        int64_t head_dim);
+int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse, void* dq, void* dk,
+                     void* dv, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q, int64_t total_k,
+                     int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t kernel_size,
+                     int64_t kernel_stride, const int64_t* strides, float sm_scale, int dtype, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
 /* ---- decode (one query per sequence over KV-cache slabs [B, slab_len, Hkv, D]) ---------------
  * strides: HOST int64 array: q(b,h) k(b,n,h) v(b,n,h) o(b,h) [+ idx(h,b,k) for the entry points
  * that read or write topk ids] = 10 or 13 values.  q/k/v strides must be multiples of 8.

@@ -1,0 +1,670 @@
+// Attention of queries over compressed keys/values (compressed_attention), forward, block
+// selection and backward.
+//
+// Tiling: a workgroup owns 16 consecutive query tokens of one sequence and one kv-head (each of
+// its 4 waves 4 tokens x the <=16 query heads of the GQA group); compressed K/V chunks of 32 keys
+// are staged once per workgroup in double-buffered LDS and shared by the 16 tokens, which see
+// almost the same causal range (key c is visible to position i iff c*stride + kernel - 1 <= i).
+// Scores are produced transposed (S^T = K Q^T) so that one lane holds one head and P^T / dS^T
+// feed the next MFMA directly; V^T and K^T fragments are read from the row-major LDS tiles with
+// ds_read_b64_tr_b16.
+//
+// Selection (replaces the dense [Hkv, T, Tc] score tensor + transform + torch.topk of the
+// reference): per token the probabilities are recomputed chunk by chunk from the final LSE,
+// summed over the group's heads, folded into block scores with the overlap weights, then the k
+// best blocks are extracted by repeated wave-wide arg-max and written in ascending order.
+#include "delta.h"
+#include "dkdv.h"
+
+struct CmpParams {
+  const void* q; const void* k; const void* v; const void* dout; void* o; void* dq; float* lse; const float* delta;
+  const int32_t* cu_q; const int32_t* cu_k;
+  int total_q, batch, Hkv, G, GT, ks, st;
+  long long qsn, qsh, ksn, ksh, vsn, vsh, osn, osh, dsn, dsh, dqsn, dqsh;
+  float qk_scale, sm_scale;
+};
+
+__device__ __forceinline__ int first_tile(const int32_t* __restrict__ cu, int b) { return (cu[b] + 15) / 16 + b; }
+static inline int64_t n_tile_slots(int64_t total_q, int64_t batch) { return (total_q + 15) / 16 + batch + 1; }
+
+struct TileInfo { int b, s0q, lq, k0, lk, i0; };
+__device__ __forceinline__ bool locate_tile(const int32_t* cu_q, const int32_t* cu_k, int batch, int slot, TileInfo& ti) {
+  int lo = 0, hi = batch;
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (first_tile(cu_q, mid) <= slot) lo = mid; else hi = mid;
+  }
+  ti.b = lo;
+  ti.s0q = cu_q[lo]; ti.lq = cu_q[lo + 1] - ti.s0q;
+  ti.k0 = cu_k[lo]; ti.lk = cu_k[lo + 1] - ti.k0;
+  ti.i0 = (slot - first_tile(cu_q, lo)) * 16;
+  return ti.i0 < ti.lq;
+}
+// number of compressed keys visible to position pos
+__device__ __forceinline__ int visible_keys(int pos, int lq, int lk, int ks, int st) {
+  if (pos >= lq || pos < ks - 1) return 0;
+  const int n = (pos - ks + 1) / st + 1;
+  return n < lk ? n : lk;
+}
+
+// stage rows [32*chunk, +32) of up to two [*, H, D] tensors into LDS tiles (zeros past lk)
+template <typename T, int D, int NTENS>
+struct Stager {
+  static constexpr int PIECES = NTENS * 32 * (D / 8);
+  static constexpr int PPT = (PIECES + 255) / 256;
+  uint4 regs[PPT];
+  __device__ __forceinline__ void fetch(const T* a, long long asn, const T* b2, long long bsn, int chunk, int lk, int tid) {
+#pragma unroll
+    for (int u = 0; u < PPT; u++) {
+      const int pc = tid + u * 256;
+      uint4 val = {0u, 0u, 0u, 0u};
+      if (pc < PIECES) {
+        const int c = pc % (D / 8), r = (pc / (D / 8)) % 32, which = pc / (D / 8) / 32;
+        const int key = chunk * 32 + r;
+        if (key < lk) val = *reinterpret_cast<const uint4*>((which == 0 ? a + (long long)key * asn : b2 + (long long)key * bsn) + 8 * c);
+      }
+      regs[u] = val;
+    }
+  }
+  __device__ __forceinline__ void stash(T (*ta)[D + 8], T (*tb)[D + 8], int tid) {
+#pragma unroll
+    for (int u = 0; u < PPT; u++) {
+      const int pc = tid + u * 256;
+      if (pc < PIECES) {
+        const int c = pc % (D / 8), r = (pc / (D / 8)) % 32, which = pc / (D / 8) / 32;
+        *reinterpret_cast<uint4*>(which == 0 ? &ta[r][8 * c] : &tb[r][8 * c]) = regs[u];
+      }
+    }
+  }
+};
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+// fragment of X^T for 16 columns starting at d0 over the 32 staged rows, in the k-order of the
+// packed score registers: slots 0..3 = rows 4*lg+r of the first 16, slots 4..7 = same of the second 16
+template <typename T, int LD>
+__device__ __forceinline__ typename Elem<T>::v8 tr_frag(const T (*tile)[LD], int d0, int li, int lg) {
+  const T* a0 = &tile[4 * lg + (li >> 2)][d0 + 4 * (li & 3)];
+  const T* a1 = &tile[16 + 4 * lg + (li >> 2)][d0 + 4 * (li & 3)];
+  s16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+  s16x4 y = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a1));
+  s16x8 z = {x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+  return __builtin_bit_cast(typename Elem<T>::v8, z);
+}
+
+// ------------------------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  using v4 = typename E::v4;
+  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8;
+  __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
+  __shared__ __attribute__((aligned(16))) T v_s[2][32][LD];
+  TileInfo ti;
+  if (!locate_tile(p.cu_q, p.cu_k, p.batch, blockIdx.x, ti)) return;
+  const int h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const int hq = gt * 16 + li;
+  const bool has_head = hq < p.G;
+  const int hh = h * p.G + (has_head ? hq : 0);
+  v8 qf[4][NK];
+  int lim[4];
+  int wave_lim = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int pos = ti.i0 + 4 * wave + j;
+    lim[j] = visible_keys(pos, ti.lq, ti.lk, p.ks, p.st);
+    wave_lim = max(wave_lim, lim[j]);
+    const bool live = has_head && pos < ti.lq;
+    const T* qp = (const T*)p.q + (long long)(ti.s0q + (pos < ti.lq ? pos : 0)) * p.qsn + (long long)hh * p.qsh + 8 * lg;
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) qf[j][kk] = live ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+  }
+  const int tile_last = min(ti.i0 + 15, ti.lq - 1);
+  const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
+  f32x4 acc[4][NDT];
+  float m[4], l[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    m[j] = -INFINITY; l[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NDT; i++) acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
+  const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
+  Stager<T, D, 2> stg;
+  if (n_chunks > 0) {
+    stg.fetch(kb, p.ksn, vb, p.vsn, 0, ti.lk, tid);
+    stg.stash(k_s[0], v_s[0], tid);
+  }
+  __syncthreads();
+  for (int ch = 0; ch < n_chunks; ch++) {
+    const int buf = ch & 1;
+    if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, vb, p.vsn, ch + 1, ti.lk, tid);
+    if (32 * ch < wave_lim) {
+      f32x4 s[4][2];
+#pragma unroll
+      for (int sub = 0; sub < 2; sub++) {
+        v8 kf[NK];
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kk = 0; kk < NK; kk++) c = E::mfma16(kf[kk], qf[j][kk], c);
+          s[j][sub] = c;
+        }
+      }
+      v8 pf[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int c = 32 * ch + 16 * sub + 4 * lg + r;
+            const float x = c < lim[j] ? s[j][sub][r] * p.qk_scale : -INFINITY;
+            s[j][sub][r] = x;
+            mloc = fmaxf(mloc, x);
+          }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+        const float m_new = fmaxf(m[j], mloc);
+        const bool dead = m_new == -INFINITY;  // nothing visible yet for this token
+        const float alpha = dead ? 1.f : fast_exp2(m[j] - m_new);
+        m[j] = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const float x = dead ? 0.f : fast_exp2(s[j][sub][r] - m_new);
+            psum += x;
+            pf[j][4 * sub + r] = (T)x;
+          }
+        l[j] = l[j] * alpha + psum;
+#pragma unroll
+        for (int i = 0; i < NDT; i++) acc[j][i] *= alpha;
+      }
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        const v8 vt = tr_frag<T, LD>(v_s[buf], 16 * dt, li, lg);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j][dt] = E::mfma16(vt, pf[j], acc[j][dt]);
+      }
+    }
+    if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], v_s[buf ^ 1], tid);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int pos = ti.i0 + 4 * wave + j;
+    float lt = l[j];
+    lt += __shfl_xor(lt, 16);
+    lt += __shfl_xor(lt, 32);
+    if (pos < ti.lq && has_head) {
+      const float inv = lt > 0.f ? 1.f / lt : 0.f;
+      T* op = (T*)p.o + (long long)(ti.s0q + pos) * p.osn + (long long)hh * p.osh + 4 * lg;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        v4 out;
+#pragma unroll
+        for (int r = 0; r < 4; r++) out[r] = (T)(acc[j][dt][r] * inv);
+        st8(op + 16 * dt, out);
+      }
+      if (lg == 0) p.lse[(long long)hh * p.total_q + ti.s0q + pos] = lt > 0.f ? m[j] + fast_log2(lt) : -INFINITY;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  using v4 = typename E::v4;
+  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8, TPW = 2;  // tokens per wave: 8-token tiles inside the 16-token slot
+  __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
+  __shared__ __attribute__((aligned(16))) T v_s[2][32][LD];
+  TileInfo ti;
+  if (!locate_tile(p.cu_q, p.cu_k, p.batch, blockIdx.x >> 1, ti)) return;
+  ti.i0 += 8 * (blockIdx.x & 1);
+  if (ti.i0 >= ti.lq) return;
+  const int h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const int hq = gt * 16 + li;
+  const bool has_head = hq < p.G;
+  const int hh = h * p.G + (has_head ? hq : 0);
+  v8 qf[TPW][NK], dof[TPW][NK];
+  int lim[TPW];
+  float l2[TPW], dl[TPW];
+  int wave_lim = 0;
+#pragma unroll
+  for (int j = 0; j < TPW; j++) {
+    const int pos = ti.i0 + TPW * wave + j;
+    lim[j] = visible_keys(pos, ti.lq, ti.lk, p.ks, p.st);
+    wave_lim = max(wave_lim, lim[j]);
+    const bool live = has_head && pos < ti.lq;
+    const long long t = ti.s0q + (pos < ti.lq ? pos : 0);
+    const T* qp = (const T*)p.q + t * p.qsn + (long long)hh * p.qsh + 8 * lg;
+    const T* dp = (const T*)p.dout + t * p.dsn + (long long)hh * p.dsh + 8 * lg;
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) {
+      qf[j][kk] = live ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+      dof[j][kk] = live ? ld16<v8>(dp + 32 * kk) : zero16<v8>();
+    }
+    l2[j] = live ? p.lse[(long long)hh * p.total_q + t] : INFINITY;
+    dl[j] = live ? p.delta[(long long)hh * p.total_q + t] : 0.f;
+  }
+  const int tile_last = min(ti.i0 + 7, ti.lq - 1);
+  const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
+  f32x4 acc[TPW][NDT];
+#pragma unroll
+  for (int j = 0; j < TPW; j++)
+#pragma unroll
+    for (int i = 0; i < NDT; i++) acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
+  const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
+  Stager<T, D, 2> stg;
+  if (n_chunks > 0) {
+    stg.fetch(kb, p.ksn, vb, p.vsn, 0, ti.lk, tid);
+    stg.stash(k_s[0], v_s[0], tid);
+  }
+  __syncthreads();
+  for (int ch = 0; ch < n_chunks; ch++) {
+    const int buf = ch & 1;
+    if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, vb, p.vsn, ch + 1, ti.lk, tid);
+    if (32 * ch < wave_lim) {
+      v8 dsf[TPW];
+#pragma unroll
+      for (int sub = 0; sub < 2; sub++) {
+        v8 kf[NK], vf[NK];
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) {
+          kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
+          vf[kk] = ld16<v8>(&v_s[buf][16 * sub + li][32 * kk + 8 * lg]);
+        }
+#pragma unroll
+        for (int j = 0; j < TPW; j++) {
+          f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kk = 0; kk < NK; kk++) {
+            s = E::mfma16(kf[kk], qf[j][kk], s);
+            dp = E::mfma16(vf[kk], dof[j][kk], dp);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int c = 32 * ch + 16 * sub + 4 * lg + r;
+            const float pr = c < lim[j] ? fast_exp2(s[r] * p.qk_scale - l2[j]) : 0.f;
+            dsf[j][4 * sub + r] = (T)(pr * (dp[r] - dl[j]) * p.sm_scale);
+          }
+        }
+      }
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        const v8 kt = tr_frag<T, LD>(k_s[buf], 16 * dt, li, lg);
+#pragma unroll
+        for (int j = 0; j < TPW; j++) acc[j][dt] = E::mfma16(kt, dsf[j], acc[j][dt]);
+      }
+    }
+    if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], v_s[buf ^ 1], tid);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < TPW; j++) {
+    const int pos = ti.i0 + TPW * wave + j;
+    if (pos < ti.lq && has_head) {
+      T* op = (T*)p.dq + (long long)(ti.s0q + pos) * p.dqsn + (long long)hh * p.dqsh + 4 * lg;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        v4 out;
+#pragma unroll
+        for (int r = 0; r < 4; r++) out[r] = (T)acc[j][dt][r];
+        st8(op + 16 * dt, out);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// block selection
+struct SelParams {
+  const void* q; const void* k; const float* lse; const int32_t* cu_q; const int32_t* cu_k; int32_t* out;
+  int total_q, batch, Hkv, G, GT, ks, st, bs, init_blocks, local_blocks, k_out, nb_cap, full_blocks;
+  long long qsn, qsh, ksn, ksh, osh, osn, osk;
+  float qk_scale;
+};
+static constexpr int SC_W = 32 + 16;  // per-token score strip: carry (<=16) + one 32-key chunk
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  constexpr int NK = D / 32, LD = D + 8;
+  __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
+  extern __shared__ float dyn[];
+  float* bs_s = dyn;                           // [16][nb_cap] block scores of the tile's tokens
+  float* sc_s = dyn + 16 * p.nb_cap;           // [4 waves][4 tokens][SC_W]
+  TileInfo ti;
+  if (!locate_tile(p.cu_q, p.cu_k, p.batch, blockIdx.x, ti)) return;
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const int a = p.ks / p.st, rr = p.bs / p.st, pad = a - 1, n_taps = a + rr - 1;
+  const int nbl = 32 / rr;  // blocks completed by one 32-key chunk
+  for (int i = tid; i < 16 * p.nb_cap; i += 256) bs_s[i] = 0.f;
+  int lim[4];
+  int wave_lim = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    lim[j] = visible_keys(ti.i0 + 4 * wave + j, ti.lq, ti.lk, p.ks, p.st);
+    wave_lim = max(wave_lim, lim[j]);
+  }
+  const int tile_last = min(ti.i0 + 15, ti.lq - 1);
+  const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
+  const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
+  float* my_sc = sc_s + wave * 4 * SC_W;
+  Stager<T, D, 1> stg;
+  __syncthreads();
+  for (int gt = 0; gt < p.GT; gt++) {
+    v8 qf[4][NK];
+    float l2[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int pos = ti.i0 + 4 * wave + j;
+      const long long t = ti.s0q + (pos < ti.lq ? pos : 0);
+      const int hq = gt * 16 + li;
+      const bool live = hq < p.G && pos < ti.lq;
+      const T* qp = (const T*)p.q + t * p.qsn + (long long)(h * p.G + (hq < p.G ? hq : 0)) * p.qsh + 8 * lg;
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) qf[j][kk] = live ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int hr = gt * 16 + 4 * lg + r;
+        l2[j][r] = (hr < p.G && pos < ti.lq) ? p.lse[(long long)(h * p.G + hr) * p.total_q + t] : INFINITY;
+      }
+    }
+    for (int i = lane; i < 4 * SC_W; i += 64) my_sc[i] = 0.f;  // carry of "chunk -1"
+    if (n_chunks > 0) {
+      stg.fetch(kb, p.ksn, kb, p.ksn, 0, ti.lk, tid);
+      stg.stash(k_s[0], k_s[0], tid);
+    }
+    __syncthreads();
+    for (int ch = 0; ch < n_chunks; ch++) {
+      const int buf = ch & 1;
+      if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, kb, p.ksn, ch + 1, ti.lk, tid);
+      if (32 * ch < wave_lim) {
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+          v8 kf[NK];
+#pragma unroll
+          for (int kk = 0; kk < NK; kk++) kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
+          const int c = 32 * ch + 16 * sub + li;  // this lane's key (column)
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < NK; kk++) s = E::mfma16(qf[j][kk], kf[kk], s);  // rows = heads 4*lg+r
+            float x = 0.f;
+            if (c < lim[j]) {
+#pragma unroll
+              for (int r = 0; r < 4; r++) x += fast_exp2(s[r] * p.qk_scale - l2[j][r]);
+            }
+            x += __shfl_xor(x, 16);
+            x += __shfl_xor(x, 32);
+            if (lg == 0) my_sc[j * SC_W + pad + 16 * sub + li] = x;
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int i = lane; i < 4 * nbl; i += 64) {
+          const int j = i / nbl, lb = i % nbl;
+          const int blk = (32 * ch) / rr + lb;
+          float v = 0.f;
+          for (int o = 0; o < n_taps; o++) {
+            const int w = min(min(o, n_taps - 1 - o), min(a - 1, rr - 1)) + 1;
+            v += (float)w * my_sc[j * SC_W + lb * rr + o];
+          }
+          if (blk < p.full_blocks && blk < p.nb_cap) bs_s[(4 * wave + j) * p.nb_cap + blk] += v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        float carry = 0.f;
+        if (lane < 4 * pad) carry = my_sc[(lane / pad) * SC_W + 32 + lane % pad];
+        __builtin_amdgcn_wave_barrier();
+        if (lane < 4 * pad) my_sc[(lane / pad) * SC_W + lane % pad] = carry;
+      }
+      if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], k_s[buf ^ 1], tid);
+      __syncthreads();
+    }
+  }
+  // forced blocks, then k best per token (value descending, index ascending), written ascending
+  for (int j = 0; j < 4; j++) {
+    const int pos = ti.i0 + 4 * wave + j;
+    if (pos >= ti.lq) continue;  // wave-uniform
+    float* row = bs_s + (4 * wave + j) * p.nb_cap;
+    const int qb = pos / p.bs;
+    const int nb = min(qb + 1, p.nb_cap);
+    for (int blk = lane; blk < nb; blk += 64)
+      if (blk < p.init_blocks || blk > qb - p.local_blocks) row[blk] = INFINITY;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int n_pick = min(p.k_out, nb);
+    int32_t* out = p.out + (long long)h * p.osh + (long long)(ti.s0q + pos) * p.osn;
+    if (n_pick == nb) {  // everything causal is selected
+      for (int i = lane; i < p.k_out; i += 64) out[(long long)i * p.osk] = i < nb ? i : -1;
+      continue;
+    }
+    for (int round = 0; round < n_pick; round++) {
+      float bv = -1.f;
+      int bi = 0x7fffffff;
+      for (int blk = lane; blk < nb; blk += 64) {
+        const float v = row[blk];
+        if (v > bv) { bv = v; bi = blk; }
+      }
+#pragma unroll
+      for (int sft = 32; sft > 0; sft >>= 1) {
+        const float ov = __shfl_xor(bv, sft);
+        const int oi = __shfl_xor(bi, sft);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+      if (lane == 0) row[bi] = -2.f;  // taken
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    int base = 0;
+    for (int blk0 = 0; blk0 < nb; blk0 += 64) {
+      const int blk = blk0 + lane;
+      const bool taken = blk < nb && row[blk] == -2.f;
+      const unsigned long long mask = __ballot(taken);
+      const int before = __popcll(mask & ((1ull << lane) - 1ull));
+      if (taken) out[(long long)(base + before) * p.osk] = blk;
+      base += __popcll(mask);
+    }
+    for (int i = n_pick + lane; i < p.k_out; i += 64) out[(long long)i * p.osk] = -1;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// dK/dV segments: blocks of 64 compressed keys per (head, sequence); their queries are the
+// contiguous range from the first position that sees the block's first key to the sequence end
+__global__ void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cu_k, int batch, int Hkv, int ks, int st,
+                                    int max_blocks, int32_t* __restrict__ cu_blk, int32_t* __restrict__ seg_begin, int32_t* __restrict__ seg_end) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int acc = 0;
+  cu_blk[0] = 0;
+  for (int b = 0; b < batch; b++) { acc += (cu_k[b + 1] - cu_k[b] + 63) / 64; cu_blk[b + 1] = acc; }
+  for (int h = 0; h < Hkv; h++) {
+    for (int g = 0; g < max_blocks; g++) { seg_begin[h * max_blocks + g] = 0; seg_end[h * max_blocks + g] = 0; }
+    for (int b = 0; b < batch; b++) {
+      const int lq = cu_q[b + 1] - cu_q[b];
+      for (int g = cu_blk[b]; g < cu_blk[b + 1]; g++) {
+        const int first_pos = (g - cu_blk[b]) * 64 * st + ks - 1;
+        seg_begin[h * max_blocks + g] = cu_q[b] + min(first_pos, lq);
+        seg_end[h * max_blocks + g] = cu_q[b] + lq;
+      }
+    }
+  }
+}
+
+struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, partial, total; int64_t max_blocks, max_items; };
+static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+  CmpBwdLayout L;
+  L.max_blocks = Tk / 64 + B;
+  const int64_t GT = (Hq / Hkv + 15) / 16;
+  (void)GT;
+  // every block's range is at most Tq tokens: ceil(Tq/CHUNK)+1 items per segment is a safe bound
+  L.max_items = Hkv * L.max_blocks * ((Tq + CHUNK_TOKENS - 1) / CHUNK_TOKENS + 1);
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
+  L.delta = take((size_t)Hq * Tq * 4);
+  L.cu_blk = take((size_t)(B + 1) * 4);
+  L.seg_begin = take((size_t)(Hkv * L.max_blocks + 1) * 4);
+  L.seg_end = take((size_t)(Hkv * L.max_blocks + 1) * 4);
+  L.chunk_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
+  L.partial = take((size_t)L.max_items * 64 * D * 4 * 2);
+  L.total = off;
+  return L;
+}
+
+// ------------------------------------------------------------------------------------------
+struct CmpArgs {
+  CmpParams p; SelParams sp; const void* o_in; void* dk; void* dv; long long dksn, dksh, dvsn, dvsh;
+  int64_t Tq, Tk, B, Hq, Hkv; char* ws; hipStream_t stream; int what;  // 0 fwd, 1 select, 2 bwd
+};
+
+template <typename T, int D>
+static int run_cmp(CmpArgs& a) {
+  const int64_t slots = n_tile_slots(a.Tq, a.B);
+  if (a.what == 0) {
+    cmp_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
+  } else if (a.what == 1) {
+    const size_t dyn = ((size_t)16 * a.sp.nb_cap + 4 * 4 * SC_W) * 4;
+    if (dyn > 64 * 1024) {
+      if (hipFuncSetAttribute((const void*)cmp_select_kernel<T, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
+        return NSA_ERR_UNSUPPORTED;
+    }
+    cmp_select_kernel<T, D><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
+  } else {
+    const CmpBwdLayout L = cmp_bwd_layout(a.Tq, a.Tk, a.B, a.Hq, a.Hkv, D);
+    float* delta = (float*)(a.ws + L.delta);
+    int32_t* cu_blk = (int32_t*)(a.ws + L.cu_blk);
+    int32_t* seg_begin = (int32_t*)(a.ws + L.seg_begin);
+    int32_t* seg_end = (int32_t*)(a.ws + L.seg_end);
+    int32_t* chunk_off = (int32_t*)(a.ws + L.chunk_off);
+    const int n_seg = (int)(a.Hkv * L.max_blocks);
+    launch_delta<T, D>((const T*)a.o_in, (const T*)a.p.dout, delta, a.Tq, a.Hq, a.p.osn, a.p.osh, a.p.dsn, a.p.dsh, a.stream);
+    cmp_segments_kernel<<<1, 64, 0, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
+    chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off);
+    DkdvParams d;
+    d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
+    d.cu_blk = cu_blk; d.seg_begin = seg_begin; d.seg_end = seg_end; d.chunk_off = chunk_off; d.queries = nullptr;
+    d.partial = (float*)(a.ws + L.partial);
+    d.total_len = (int)a.Tq; d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;
+    d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st;
+    d.qsn = a.p.qsn; d.qsh = a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = a.p.dsn; d.dsh = a.p.dsh;
+    d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
+    dkdv_kernel<T, D, 64, true><<<(unsigned)L.max_items, 256, 0, a.stream>>>(d);
+    dkdv_reduce_kernel<T, D, 64><<<(unsigned)n_seg, 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
+                                                                       (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
+    a.p.delta = delta;
+    cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
+  }
+  return nsa_check_launch();
+}
+
+static int cmp_dispatch(CmpArgs& a, int64_t head_dim, int dtype) {
+#define CALL(T, D) run_cmp<T, D>(a)
+  switch (head_dim) {
+    case 32: return dtype == NSA_BF16 ? CALL(__bf16, 32) : CALL(_Float16, 32);
+    case 64: return dtype == NSA_BF16 ? CALL(__bf16, 64) : CALL(_Float16, 64);
+    case 96: return dtype == NSA_BF16 ? CALL(__bf16, 96) : CALL(_Float16, 96);
+    case 128: return dtype == NSA_BF16 ? CALL(__bf16, 128) : CALL(_Float16, 128);
+  }
+#undef CALL
+  return NSA_ERR_UNSUPPORTED;
+}
+
+static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, const int32_t* cu_q, const int32_t* cu_k, int64_t Tq,
+                      int64_t Tk, int64_t B, int64_t Hq, int64_t Hkv, int64_t ks, int64_t st, const int64_t* strides, float sm_scale,
+                      int dtype, void* stream) {
+  if (!q || !k || !cu_q || !cu_k || !strides || Tq <= 0 || Tk < 0 || B <= 0 || Hkv <= 0 || Hq % Hkv != 0 || ks <= 0 || st <= 0) return NSA_ERR_BAD_ARG;
+  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  for (int i = 0; i < 6; i++) if (strides[i] % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 != 0) return NSA_ERR_UNSUPPORTED;
+  CmpParams& p = a.p;
+  p.q = q; p.k = k; p.v = v; p.cu_q = cu_q; p.cu_k = cu_k; p.total_q = (int)Tq; p.batch = (int)B; p.Hkv = (int)Hkv;
+  p.G = (int)(Hq / Hkv); p.GT = (p.G + 15) / 16; p.ks = (int)ks; p.st = (int)st;
+  p.qsn = strides[0]; p.qsh = strides[1]; p.ksn = strides[2]; p.ksh = strides[3]; p.vsn = strides[4]; p.vsh = strides[5];
+  p.qk_scale = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale;
+  p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr;
+  a.Tq = Tq; a.Tk = Tk; a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.stream = (hipStream_t)stream; a.ws = nullptr;
+  return NSA_OK;
+}
+
+extern "C" int nsa_cmp_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens_q,
+                                const int32_t* cu_seqlens_k, int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads,
+                                int64_t num_kv_heads, int64_t head_dim, int64_t kernel_size, int64_t kernel_stride,
+                                const int64_t* strides, float sm_scale, int dtype, void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, v, cu_seqlens_q, cu_seqlens_k, total_q, total_k, batch, num_q_heads, num_kv_heads, kernel_size, kernel_stride, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!v || !o || !lse || strides[6] % 4 != 0 || strides[7] % 4 != 0 || (uintptr_t)o % 8 != 0) return NSA_ERR_BAD_ARG;
+  a.p.o = o; a.p.lse = lse; a.p.osn = strides[6]; a.p.osh = strides[7];
+  a.what = 0;
+  return cmp_dispatch(a, head_dim, dtype);
+}
+
+extern "C" int nsa_cmp_attn_select(const void* q, const void* k, const float* lse, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                   int32_t* out_topk_idx, int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads,
+                                   int64_t num_kv_heads, int64_t head_dim, int64_t kernel_size, int64_t kernel_stride,
+                                   int64_t block_size, int64_t k_out, int64_t max_seqlen_q, int64_t init_blocks, int64_t local_blocks,
+                                   const int64_t* strides, float sm_scale, int dtype, void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, k, cu_seqlens_q, cu_seqlens_k, total_q, total_k, batch, num_q_heads, num_kv_heads, kernel_size, kernel_stride, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!lse || !out_topk_idx || k_out <= 0 || max_seqlen_q <= 0) return NSA_ERR_BAD_ARG;
+  if (kernel_size % kernel_stride != 0 || block_size % kernel_size != 0) return NSA_ERR_BAD_ARG;
+  const int64_t rr = block_size / kernel_stride, pad = kernel_size / kernel_stride - 1;
+  if (rr > 32 || 32 % rr != 0 || pad > 16) return NSA_ERR_UNSUPPORTED;
+  const int64_t nb = (max_seqlen_q + block_size - 1) / block_size;
+  if (k_out > nb) return NSA_ERR_BAD_ARG;
+  if (((size_t)16 * nb + 4 * 4 * SC_W) * 4 > 140 * 1024) return NSA_ERR_UNSUPPORTED;  // block-score strip must fit LDS
+  SelParams& s = a.sp;
+  s.q = q; s.k = k; s.lse = lse; s.cu_q = cu_seqlens_q; s.cu_k = cu_seqlens_k; s.out = out_topk_idx;
+  s.total_q = (int)total_q; s.batch = (int)batch; s.Hkv = (int)num_kv_heads; s.G = a.p.G; s.GT = a.p.GT; s.ks = (int)kernel_size;
+  s.st = (int)kernel_stride; s.bs = (int)block_size; s.init_blocks = (int)init_blocks; s.local_blocks = (int)local_blocks;
+  s.k_out = (int)k_out; s.nb_cap = (int)nb; s.full_blocks = (int)(max_seqlen_q / block_size);
+  s.qsn = strides[0]; s.qsh = strides[1]; s.ksn = strides[2]; s.ksh = strides[3]; s.osh = strides[6]; s.osn = strides[7]; s.osk = strides[8];
+  s.qk_scale = sm_scale * NSA_LOG2E;
+  a.what = 1;
+  return cmp_dispatch(a, head_dim, dtype);
+}
+
+extern "C" size_t nsa_cmp_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                                   int64_t head_dim) {
+  return cmp_bwd_layout(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim).total;
+}
+
+extern "C" int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse, void* dq,
+                                void* dk, void* dv, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q,
+                                int64_t total_k, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                int64_t kernel_size, int64_t kernel_stride, const int64_t* strides, float sm_scale, int dtype,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, v, cu_seqlens_q, cu_seqlens_k, total_q, total_k, batch, num_q_heads, num_kv_heads, kernel_size, kernel_stride, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!v || !o || !dout || !lse || !dq || !dk || !dv || !workspace) return NSA_ERR_BAD_ARG;
+  for (int i = 6; i < 10; i++) if (strides[i] % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  for (int i = 10; i < 16; i++) if (strides[i] % 4 != 0) return NSA_ERR_UNSUPPORTED;
+  if (((uintptr_t)o | (uintptr_t)dout) % 16 != 0 || ((uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) % 8 != 0 || (uintptr_t)workspace % 256 != 0) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_cmp_attn_bwd_workspace_bytes(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
+  a.o_in = o; a.p.dout = dout; a.p.lse = (float*)lse; a.p.dq = dq; a.dk = dk; a.dv = dv;
+  a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
+  a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
+  a.ws = (char*)workspace;
+  a.what = 2;
+  return cmp_dispatch(a, head_dim, dtype);
+}

@@ -15,6 +15,8 @@
 #include <rocprim/device/device_radix_sort.hpp>
 
 #include "block_transpose.h"
+#include "delta.h"
+#include "dkdv.h"
 
 // ------------------------------------------------------------------------------------------
 // workspace carving (host and entry point must agree)
@@ -23,8 +25,6 @@ struct BwdLayout {
   size_t sort_tmp_bytes;
   int64_t max_blocks, n_pairs, max_items, n_slots;
 };
-
-static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -56,33 +56,6 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.partial = take((size_t)L.max_items * bs * D * 4 * 2);
   L.total = off;
   return L;
-}
-
-// ------------------------------------------------------------------------------------------
-// pass 1: delta
-template <typename T, int D>
-__global__ __launch_bounds__(256) void delta_kernel(const T* __restrict__ o, const T* __restrict__ dout, float* __restrict__ delta,
-                                                    int total_len, int Hq, long long osn, long long osh, long long dsn, long long dsh) {
-  using v8 = typename Elem<T>::v8;
-  constexpr int LPR = D / 8;                       // lanes per row (16-byte pieces)
-  constexpr int LPR2 = LPR <= 4 ? 4 : (LPR <= 8 ? 8 : 16);
-  const int sub = threadIdx.x % LPR2;
-  const long long row = (long long)blockIdx.x * (256 / LPR2) + threadIdx.x / LPR2;
-  const bool live = row < (long long)total_len * Hq;
-  float acc = 0.f;
-  int t = 0, h = 0;
-  if (live) {
-    t = (int)(row / Hq); h = (int)(row % Hq);
-    if (sub < LPR) {
-      v8 a = ld16<v8>(o + (long long)t * osn + (long long)h * osh + 8 * sub);
-      v8 b = ld16<v8>(dout + (long long)t * dsn + (long long)h * dsh + 8 * sub);
-#pragma unroll
-      for (int i = 0; i < 8; i++) acc += (float)a[i] * (float)b[i];
-    }
-  }
-#pragma unroll
-  for (int s = LPR2 / 2; s > 0; s >>= 1) acc += __shfl_xor(acc, s);
-  if (live && sub == 0) delta[(long long)h * total_len + t] = acc;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -127,251 +100,6 @@ __global__ __launch_bounds__(256) void segment_offsets_kernel(const uint32_t* __
     if (keys[mid] < (uint32_t)j) lo = mid + 1; else hi = mid;
   }
   seg_off[j] = (int32_t)lo;
-}
-
-// chunk_off = exclusive scan of ceil(count/CHUNK_TOKENS) over segments (single workgroup).
-__global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* __restrict__ seg_off, int n_seg, int32_t* __restrict__ chunk_off) {
-  __shared__ int part[1024];
-  const int tid = threadIdx.x;
-  const int per = (n_seg + 1023) / 1024;
-  const int j0 = tid * per, j1 = min(n_seg, j0 + per);
-  int s = 0;
-  for (int j = j0; j < j1; j++) s += (seg_off[j + 1] - seg_off[j] + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
-  part[tid] = s;
-  __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {
-    int v = tid >= d ? part[tid - d] : 0;
-    __syncthreads();
-    part[tid] += v;
-    __syncthreads();
-  }
-  int run = part[tid] - s;
-  for (int j = j0; j < j1; j++) {
-    chunk_off[j] = run;
-    run += (seg_off[j + 1] - seg_off[j] + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
-  }
-  if (tid == 1023) chunk_off[n_seg] = part[1023];
-}
-
-// ------------------------------------------------------------------------------------------
-// pass 3: dK / dV
-struct DkdvParams {
-  const void* q; const void* k; const void* v; const void* dout; const float* lse; const float* delta;
-  const int32_t* cu; const int32_t* cu_blk; const int32_t* seg_off; const int32_t* chunk_off; const int32_t* queries;
-  float* partial;
-  int total_len, batch, Hkv, G, GT, max_blocks, n_seg;
-  long long qsn, qsh, ksn, ksh, vsn, vsh, dsn, dsh;
-  float qk_scale, sm_scale;
-};
-
-template <typename T, int D, int BS>
-__global__ __launch_bounds__(BS >= 64 ? 256 : 128) void dkdv_kernel(DkdvParams p) {
-  using E = Elem<T>;
-  using v8 = typename E::v8;
-  constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16;
-  constexpr int NW = NSUB < 4 ? NSUB : 4;     // waves per workgroup
-  constexpr int KT = NSUB / NW;               // 16-key tiles per wave
-  constexpr int NT = NW * 64;
-  constexpr int LD = D + 8;                   // padded LDS row (elements)
-  __shared__ __attribute__((aligned(16))) T q_s[2][2][16][LD];
-  __shared__ __attribute__((aligned(16))) T do_s[2][2][16][LD];
-  __shared__ float lse_s[2][32], delta_s[2][32];
-  __shared__ int pos_s[2][2];
-
-  const int total_items = p.chunk_off[p.n_seg];
-  const int item = blockIdx.x;
-  if (item >= total_items) return;
-  // segment (head, global block) that owns this work item
-  int lo = 0, hi = p.n_seg;  // chunk_off[lo] <= item < chunk_off[hi]
-  while (hi - lo > 1) {
-    int mid = (lo + hi) >> 1;
-    if (p.chunk_off[mid] <= item) lo = mid; else hi = mid;
-  }
-  const int seg = lo;
-  const int h = seg / p.max_blocks, gb = seg % p.max_blocks;
-  const int b = find_sequence(p.cu_blk, p.batch, gb);
-  const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
-  const int key0 = (gb - p.cu_blk[b]) * BS;
-  const int first = p.seg_off[seg] + (item - p.chunk_off[seg]) * CHUNK_TOKENS;
-  const int n_tok = min(CHUNK_TOKENS, p.seg_off[seg + 1] - first);
-  const int n_rg = n_tok * p.GT;              // row groups (token, head tile) in this chunk
-  const int n_step = (n_rg + 1) / 2;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int li = lane & 15, lg = lane >> 4;
-
-  // stationary operands: this wave's keys of K and V, B-operand layout (column = key)
-  v8 kf[KT][NK], vf[KT][NK];
-#pragma unroll
-  for (int j = 0; j < KT; j++) {
-    int row = key0 + 16 * (wave * KT + j) + li;
-    row = row < len ? row : len - 1;
-    const T* kp = (const T*)p.k + (long long)(s0 + row) * p.ksn + (long long)h * p.ksh + 8 * lg;
-    const T* vp = (const T*)p.v + (long long)(s0 + row) * p.vsn + (long long)h * p.vsh + 8 * lg;
-#pragma unroll
-    for (int kk = 0; kk < NK; kk++) { kf[j][kk] = ld16<v8>(kp + 32 * kk); vf[j][kk] = ld16<v8>(vp + 32 * kk); }
-  }
-  f32x4 dk[KT][NDT], dv[KT][NDT];
-#pragma unroll
-  for (int j = 0; j < KT; j++)
-#pragma unroll
-    for (int i = 0; i < NDT; i++) { dk[j][i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[j][i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-
-  // staging: 2 row groups x 16 heads x D elements for each of Q and dO = 2*2*16*D/8 16-byte pieces
-  constexpr int PIECES = 2 * 2 * 16 * (D / 8);
-  constexpr int PPT = (PIECES + NT - 1) / NT;
-  uint4 stage[PPT];
-  float st_lse = 0.f, st_delta = 0.f;
-  int st_pos = 0;
-
-  auto fetch = [&](int step) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * NT;
-      uint4 val = {0u, 0u, 0u, 0u};
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = (pc / (D / 8) / 16) % 2, which = pc / (D / 8) / 32;
-        const int r = step * 2 + rg;
-        if (r < n_rg) {
-          const int t = p.queries[first + r / p.GT];
-          const int hq = (r % p.GT) * 16 + hd;
-          if (hq < p.G) {
-            const T* src = which == 0 ? (const T*)p.q + (long long)t * p.qsn + (long long)(h * p.G + hq) * p.qsh
-                                      : (const T*)p.dout + (long long)t * p.dsn + (long long)(h * p.G + hq) * p.dsh;
-            val = *reinterpret_cast<const uint4*>(src + 8 * c);
-          }
-        }
-      }
-      stage[u] = val;
-    }
-    if (tid < 32) {
-      const int rg = tid >> 4, hd = tid & 15;
-      const int r = step * 2 + rg;
-      st_lse = INFINITY; st_delta = 0.f; st_pos = -1;
-      if (r < n_rg) {
-        const int t = p.queries[first + r / p.GT];
-        const int hq = (r % p.GT) * 16 + hd;
-        st_pos = t - s0;
-        if (hq < p.G) {
-          st_lse = p.lse[(long long)(h * p.G + hq) * p.total_len + t];
-          st_delta = p.delta[(long long)(h * p.G + hq) * p.total_len + t];
-        }
-      }
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * NT;
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = (pc / (D / 8) / 16) % 2, which = pc / (D / 8) / 32;
-        T* dst = which == 0 ? &q_s[buf][rg][hd][8 * c] : &do_s[buf][rg][hd][8 * c];
-        *reinterpret_cast<uint4*>(dst) = stage[u];
-      }
-    }
-    if (tid < 32) {
-      lse_s[buf][tid] = st_lse;
-      delta_s[buf][tid] = st_delta;
-      if ((tid & 15) == 0) pos_s[buf][tid >> 4] = st_pos;
-    }
-  };
-
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  for (int step = 0; step < n_step; step++) {
-    const int buf = step & 1;
-    if (step + 1 < n_step) fetch(step + 1);
-
-    // S = Q K^T and dP = dO V^T for this wave's keys; lane holds column key=li, rows 4*lg+r of each token
-    v8 pf[KT], dsf[KT];
-#pragma unroll
-    for (int j = 0; j < KT; j++) {
-      const int key = key0 + 16 * (wave * KT + j) + li;
-#pragma unroll
-      for (int tk = 0; tk < 2; tk++) {
-        f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < NK; kk++) {
-          v8 qa = ld16<v8>(&q_s[buf][tk][li][32 * kk + 8 * lg]);
-          v8 da = ld16<v8>(&do_s[buf][tk][li][32 * kk + 8 * lg]);
-          s = E::mfma16(qa, kf[j][kk], s);
-          dp = E::mfma16(da, vf[j][kk], dp);
-        }
-        const int pos = pos_s[buf][tk];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const float l2 = lse_s[buf][tk * 16 + 4 * lg + r];
-          const float dl = delta_s[buf][tk * 16 + 4 * lg + r];
-          const float pr = key <= pos ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
-          pf[j][tk * 4 + r] = (T)pr;
-          dsf[j][tk * 4 + r] = (T)(pr * (dp[r] - dl) * p.sm_scale);
-        }
-      }
-    }
-    // dV^T[d][key] += dO^T[d][row] P[row][key];  dK^T[d][key] += Q^T[d][row] dS[row][key]
-    // transposed fragments come from LDS: lane j of a 16-lane group addresses the 4-element
-    // chunk (row 4*lg + j/4, columns 16*dt + 4*(j%4)) and receives column li of those 4 rows.
-#pragma unroll
-    for (int dt = 0; dt < NDT; dt++) {
-      typedef short s16x4 __attribute__((ext_vector_type(4)));
-      typedef short s16x8 __attribute__((ext_vector_type(8)));
-      s16x8 qt, dot;
-#pragma unroll
-      for (int tk = 0; tk < 2; tk++) {
-        const T* qa = &q_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
-        const T* da = &do_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
-        s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(qa));
-        s16x4 c = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(da));
-#pragma unroll
-        for (int r = 0; r < 4; r++) { qt[tk * 4 + r] = a[r]; dot[tk * 4 + r] = c[r]; }
-      }
-      const v8 qtf = __builtin_bit_cast(v8, qt), dotf = __builtin_bit_cast(v8, dot);
-#pragma unroll
-      for (int j = 0; j < KT; j++) {
-        dv[j][dt] = E::mfma16(dotf, pf[j], dv[j][dt]);
-        dk[j][dt] = E::mfma16(qtf, dsf[j], dk[j][dt]);
-      }
-    }
-    if (step + 1 < n_step) stash(buf ^ 1);
-    __syncthreads();
-  }
-  // partial[item][0 = dK, 1 = dV][key][d], fp32
-  float* out = p.partial + (long long)item * 2 * BS * D;
-#pragma unroll
-  for (int j = 0; j < KT; j++) {
-    const int kl = 16 * (wave * KT + j) + li;
-#pragma unroll
-    for (int dt = 0; dt < NDT; dt++) {
-      *reinterpret_cast<f32x4*>(out + (long long)kl * D + 16 * dt + 4 * lg) = dk[j][dt];
-      *reinterpret_cast<f32x4*>(out + (long long)(BS + kl) * D + 16 * dt + 4 * lg) = dv[j][dt];
-    }
-  }
-}
-
-template <typename T, int D, int BS>
-__global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restrict__ partial, const int32_t* __restrict__ chunk_off,
-                                                          const int32_t* __restrict__ cu, const int32_t* __restrict__ cu_blk,
-                                                          int batch, int max_blocks, T* __restrict__ dk, T* __restrict__ dv,
-                                                          long long dksn, long long dksh, long long dvsn, long long dvsh) {
-  const int seg = blockIdx.x;
-  const int h = seg / max_blocks, gb = seg % max_blocks;
-  if (gb >= cu_blk[batch]) return;
-  const int b = find_sequence(cu_blk, batch, gb);
-  const int s0 = cu[b], len = cu[b + 1] - s0;
-  const int key0 = (gb - cu_blk[b]) * BS;
-  const int c0 = chunk_off[seg], c1 = chunk_off[seg + 1];
-  for (int i = threadIdx.x; i < 2 * BS * (D / 4); i += 256) {
-    const int which = i / (BS * (D / 4)), key = (i / (D / 4)) % BS, d4 = i % (D / 4);
-    if (key0 + key >= len) continue;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c = c0; c < c1; c++) acc += *reinterpret_cast<const f32x4*>(partial + ((long long)c * 2 + which) * BS * D + (long long)key * D + 4 * d4);
-    typename Elem<T>::v4 o;
-#pragma unroll
-    for (int r = 0; r < 4; r++) o[r] = (T)acc[r];
-    T* dst = which == 0 ? dk + (long long)(s0 + key0 + key) * dksn + (long long)h * dksh : dv + (long long)(s0 + key0 + key) * dvsn + (long long)h * dvsh;
-    st8(dst + 4 * d4, o);
-  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -499,7 +227,7 @@ static int build_reverse_index(const BwdArgs& a, const BwdLayout& L) {
   if (rocprim::radix_sort_pairs(ws + L.sort_tmp, tmp, keys_in, keys_out, vals_in, vals_out, (size_t)L.n_pairs, 0u, bits, a.stream) != hipSuccess)
     return NSA_ERR_LAUNCH;
   segment_offsets_kernel<<<(n_seg + 1 + 255) / 256, 256, 0, a.stream>>>(keys_out, L.n_pairs, n_seg, seg_off);
-  chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_off, n_seg, chunk_off);
+  chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_off, seg_off + 1, n_seg, chunk_off);
   return nsa_check_launch();
 }
 
@@ -510,12 +238,8 @@ static int run_bwd(const BwdArgs& a) {
   float* delta = (float*)(ws + L.delta);
   const int G = (int)(a.Hq / a.Hkv), GT = (G + 15) / 16;
   const int n_seg = (int)(a.Hkv * L.max_blocks);
-  if (a.phases & NSA_BWD_PHASE_PREP) {
-    constexpr int LPR = D / 8, LPR2 = LPR <= 4 ? 4 : (LPR <= 8 ? 8 : 16);
-    const long long rows = (long long)a.T * a.Hq;
-    delta_kernel<T, D><<<(unsigned)((rows + 256 / LPR2 - 1) / (256 / LPR2)), 256, 0, a.stream>>>(
-        (const T*)a.o, (const T*)a.dout, delta, (int)a.T, (int)a.Hq, a.osn, a.osh, a.dsn, a.dsh);
-  }
+  if (a.phases & NSA_BWD_PHASE_PREP)
+    launch_delta<T, D>((const T*)a.o, (const T*)a.dout, delta, a.T, a.Hq, a.osn, a.osh, a.dsn, a.dsh, a.stream);
   if (a.phases & NSA_BWD_PHASE_PREP) {
     int rc = build_reverse_index(a, L);
     if (rc != NSA_OK) return rc;
@@ -527,14 +251,14 @@ static int run_bwd(const BwdArgs& a) {
   if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;
     p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.cu = a.cu;
-    p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_off = (const int32_t*)(ws + L.seg_off);
+    p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_begin = (const int32_t*)(ws + L.seg_off); p.seg_end = p.seg_begin + 1;
     p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.vals_out);
     p.partial = (float*)(ws + L.partial);
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
     p.qsn = a.qsn; p.qsh = a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = a.dsn; p.dsh = a.dsh;
-    p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
+    p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1;
     constexpr int NT = (BS / 16 < 4 ? BS / 16 : 4) * 64;
-    dkdv_kernel<T, D, BS><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
+    dkdv_kernel<T, D, BS, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
     dkdv_reduce_kernel<T, D, BS><<<(unsigned)n_seg, 256, 0, a.stream>>>(
         p.partial, p.chunk_off, a.cu, p.cu_blk, (int)a.B, (int)L.max_blocks, (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
   }

@@ -32,6 +32,10 @@ _SIGNATURES = {
     "nsa_topk_decode": (c_int, [P] * 6 + [I] * 7 + [P, F, c_int, P, Z, P]),
     "nsa_cmp_decode_workspace_bytes": (Z, [I] * 5),
     "nsa_cmp_decode": (c_int, [P] * 7 + [I] * 12 + [P, F, c_int, P, Z, P]),
+    "nsa_cmp_attn_fwd": (c_int, [P] * 7 + [I] * 8 + [P, F, c_int, P]),
+    "nsa_cmp_attn_select": (c_int, [P] * 6 + [I] * 13 + [P, F, c_int, P]),
+    "nsa_cmp_attn_bwd_workspace_bytes": (Z, [I] * 6),
+    "nsa_cmp_attn_bwd": (c_int, [P] * 11 + [I] * 8 + [P, F, c_int, P, Z, P]),
 }
 
 

@@ -1,0 +1,93 @@
+"""GPU parity of compressed_attention (output, gradients, selected block ids) against the oracle."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close
+from native_sparse_attention.ops import avgpool_compress, compressed_attention
+from native_sparse_attention.testing import cu_from_lens
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # lens, Hq, Hkv, d, ks, st, bs, topk, dtype
+    ([1000, 4000, 8192], 32, 8, 96, 32, 16, 64, 16, torch.float16),   # the reference's own test shape
+    ([100, 257, 512], 4, 2, 32, 32, 16, 64, 4, torch.bfloat16),
+    ([1024, 3000], 64, 4, 128, 32, 16, 64, 16, torch.bfloat16),        # benchmark head layout
+    ([40, 700, 31, 65], 6, 2, 64, 32, 16, 64, 5, torch.bfloat16),      # G=3, a sequence with no compressed token
+    ([900], 40, 2, 64, 64, 16, 128, 4, torch.float16),                 # G=20 (two head tiles), ks 64 / bs 128
+    ([2100], 16, 1, 128, 32, 32, 64, 8, torch.bfloat16),               # non-overlapping windows (pad 0)
+]
+
+
+def _inputs(lens, Hq, Hkv, d, ks, st, dtype, device, seed=0):
+    g = torch.Generator(device=device).manual_seed(seed)
+    cu = cu_from_lens(lens, device)
+    T = int(cu[-1])
+    q = torch.randn(T, Hq, d, generator=g, device=device).to(dtype)
+    kx = torch.randn(T, Hkv, d, generator=g, device=device).to(dtype)
+    vx = torch.randn(T, Hkv, d, generator=g, device=device).to(dtype)
+    ck, cuk = oracle.avgpool_compress(kx.float(), None, cu, ks, st)
+    cv, _ = oracle.avgpool_compress(vx.float(), None, cu, ks, st)
+    # spread the compressed keys so that attention is not nearly uniform
+    return q, (ck * 4).to(dtype), (cv * 4).to(dtype), cu, cuk
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv,d,ks,st,bs,topk,dtype", CASES)
+def test_forward_backward_and_selection(device, lens, Hq, Hkv, d, ks, st, bs, topk, dtype):
+    print("case", lens, Hq, Hkv, d, ks, st, bs, topk, dtype, flush=True)
+    q, ck, cv, cu, cuk = _inputs(lens, Hq, Hkv, d, ks, st, dtype, device)
+    q1, k1, v1 = (x.clone().requires_grad_() for x in (q, ck, cv))
+    o, idx = compressed_attention(q1, k1, v1, ks, st, bs, topk, cu, cuk)
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, ck, cv))
+    want, want_idx, bscore = oracle.compressed_attention(qf, kf, vf, ks, st, bs, topk, cu, cuk, return_scores=True)
+    assert_close(o, want, "o")
+    g = torch.Generator(device=device).manual_seed(7)
+    do = torch.randn(o.shape, generator=g, device=device).to(dtype)
+    o.backward(do)
+    want.backward(do.float())
+    assert_close(q1.grad, qf.grad, "dq", rel_to=qf.grad.abs().max().item())
+    assert_close(k1.grad, kf.grad, "dk", rel_to=kf.grad.abs().max().item())
+    assert_close(v1.grad, vf.grad, "dv", rel_to=vf.grad.abs().max().item())
+
+    # selection: shape/dtype, structure on every row, bit-exact wherever the oracle's decision margin is clear
+    kk = min(topk, math.ceil(max(lens) / bs))
+    assert idx.shape == (Hkv, int(cu[-1]), kk) and idx.dtype == torch.int32
+    pos = torch.cat([torch.arange(L, device=device) for L in lens])
+    qb = pos // bs
+    valid = idx >= 0
+    assert (valid.sum(-1) == torch.minimum(qb + 1, torch.tensor(kk, device=device))[None]).all()
+    assert ((idx <= qb[None, :, None]) | ~valid).all()
+    srt = torch.where(valid, idx, torch.full_like(idx, 1 << 30))
+    assert (srt[..., 1:] > srt[..., :-1]).logical_or(~valid[..., 1:]).all()          # ascending, -1 right-padded
+    assert (idx[..., 0] == 0).all()                                                    # init block
+    own = (idx == qb[None, :, None]).any(-1)
+    assert own.all()                                                                   # local block
+    # margin between the worst selected and the best rejected causal, unforced block score
+    causal = torch.arange(bscore.shape[-1], device=device)[None, None] <= qb[None, :, None]
+    sc = torch.where(causal & torch.isfinite(bscore), bscore, torch.full_like(bscore, float("nan")))
+    sel = torch.zeros_like(bscore, dtype=torch.bool)
+    sel.scatter_(2, want_idx.clamp(min=0).long(), True)
+    sel &= causal
+    worst_in = torch.where(sel, sc, torch.full_like(sc, float("inf"))).nan_to_num(float("inf")).amin(-1)
+    best_out = torch.where(~sel & causal, sc, torch.full_like(sc, float("-inf"))).nan_to_num(float("-inf")).amax(-1)
+    clear = (worst_in - best_out) > 1e-3
+    exact = (idx == want_idx).all(-1)
+    assert exact[clear].all(), "%d rows with a clear margin differ" % int((~exact[clear]).sum())
+    overlap = (idx[..., :, None] == want_idx[..., None, :]).any(-1).float().mean().item()
+    print("rows with clear margin: %.1f%%, exact rows overall: %.2f%%, id overlap %.4f"
+          % (100 * clear.float().mean().item(), 100 * exact.float().mean().item(), overlap), flush=True)
+    assert overlap > 0.97
+
+
+def test_topk_disabled_and_given_max_seqlens(device):
+    q, ck, cv, cu, cuk = _inputs([300, 200], 8, 2, 64, 32, 16, torch.bfloat16, device)
+    with pytest.warns(UserWarning):
+        o, idx = compressed_attention(q, ck, cv, 32, 16, 64, -1, cu, cuk, 300, 17)
+    assert idx is None
+    want, _ = oracle.compressed_attention(q.float(), ck.float(), cv.float(), 32, 16, 64, -1, cu, cuk)
+    assert_close(o, want, "o")
+    with pytest.raises(AssertionError):
+        compressed_attention(q, ck, cv, 32, 16, 64, 2, cu, cuk)          # topk < init_blocks + local_blocks
