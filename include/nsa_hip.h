@@ -105,6 +105,24 @@ int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* dx, void* d
                  int64_t dy_stride_n, int64_t dy_stride_h, int64_t dx_stride_n, int64_t dx_stride_h, int64_t w_stride_h,
                  int64_t dw_stride_h, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- linear_compress ----------------------------------------------------------------------------
+ * Forward: replaces linear_compress_fwd_kernel (native_sparse_attention/ops/triton/linear_compress.py:27-136,
+ * launched at :379-410).  x [total_x,H,D]; w [H, kernel_size*D, D] contiguous; y [total_y,H,D].
+ */
+int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
+                            int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
+                            int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
+                            int64_t y_stride_n, int64_t y_stride_h, int dtype, void* stream);
+/* Backward: replaces linear_compress_bwd_kernel and its fp32 atomic adds (:140-306, launched at
+ * :449-480).  dx [total_x,H,D]; dw [H, kernel_size*D, D] contiguous, both in the dtype of x.
+ * Gather formulation, no atomics: reproducible.
+ */
+int nsa_linear_compress_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, const int32_t* cu_seqlens,
+                            const int32_t* y_cu_seqlens, int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads,
+                            int64_t head_dim, int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
+                            int64_t dy_stride_n, int64_t dy_stride_h, int64_t dx_stride_n, int64_t dx_stride_h, int dtype,
+                            void* stream);
+
 /* ---- compressed_attention --------------------------------------------------------------------
  * Forward: replaces forward_kernel launched from _compressed_attention_fwd
  * (native_sparse_attention/ops/triton/compressed_attention.py:538-640).  q,o [Tq,Hq,D];

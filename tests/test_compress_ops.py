@@ -78,3 +78,46 @@ def test_pool_asserts(device):
         weightedpool_compress(x, torch.ones(2, 32, device=device), cu, 32, 16)          # dtype mismatch
     with pytest.raises(AssertionError):
         weightedpool_compress(x, torch.ones(2, 24, device=device).bfloat16(), cu, 24, 8)  # kernel size set
+
+
+LINEAR_CASES = [
+    # lens, H, d, ks, st, dtype
+    ([1024, 7168, 8192], 4, 128, 32, 16, torch.bfloat16),         # BASELINE config 1 shape
+    ([12, 100, 257, 64], 2, 64, 32, 16, torch.float16),
+    ([300, 75], 3, 96, 16, 16, torch.bfloat16),
+    ([500], 2, 192, 32, 16, torch.float16),                        # the reference's d=192 smoke shape
+    ([900, 130], 1, 32, 64, 32, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("lens,H,d,ks,st,dtype", LINEAR_CASES)
+def test_linear_compress_forward_backward(device, lens, H, d, ks, st, dtype):
+    from native_sparse_attention.ops import linear_compress
+    print("case", lens, H, d, ks, st, dtype, flush=True)
+    g = torch.Generator(device=device).manual_seed(0)
+    cu = cu_from_lens(lens, device)
+    x = torch.randn(int(cu[-1]), H, d, generator=g, device=device).to(dtype)
+    w = (torch.randn(H, ks * d, d, generator=g, device=device) / (ks * d) ** 0.5).to(dtype)
+    pe = (0.02 * torch.randn(H, ks, d, generator=g, device=device)).to(dtype)
+    x1, w1, pe1 = (t.clone().requires_grad_() for t in (x, w, pe))
+    y, ycu = linear_compress(x1, w1, cu, ks, st, pe1)
+    xf, wf, pef = (t.float().requires_grad_() for t in (x, w, pe))
+    want, want_cu = oracle.linear_compress(xf, wf, cu, ks, st, pef)
+    assert torch.equal(ycu.cpu(), want_cu.cpu()) and y.dtype == dtype
+    # |y| reaches ~5 here: half an ulp of a bf16 output at that magnitude is already 1.6e-2, so the
+    # bound scales with the largest reference magnitude
+    assert_close(y, want, "y", rel_to=want.abs().max().item())
+    dy = torch.randn(y.shape, generator=g, device=device).to(dtype)
+    y.backward(dy)
+    want.backward(dy.float())
+    assert_close(x1.grad, xf.grad, "dx", rel_to=xf.grad.abs().max().item())
+    assert_close(w1.grad, wf.grad, "dw", rel_to=wf.grad.abs().max().item())
+    assert_close(pe1.grad, pef.grad, "dpe", rel_to=pef.grad.abs().max().item())
+    # reproducible: no atomics anywhere in the backward
+    x2, w2 = x.clone().requires_grad_(), w.clone().requires_grad_()
+    y2, _ = linear_compress(x2, w2, cu, ks, st)
+    y2.backward(dy)
+    x3, w3 = x.clone().requires_grad_(), w.clone().requires_grad_()
+    y3, _ = linear_compress(x3, w3, cu, ks, st)
+    y3.backward(dy)
+    assert torch.equal(x2.grad, x3.grad) and torch.equal(w2.grad, w3.grad)
