@@ -20,6 +20,7 @@ struct CmpParams {
   const void* q; const void* k; const void* v; const void* dout; void* o; void* dq; float* lse; const float* delta;
   const int32_t* cu_q; const int32_t* cu_k;
   int total_q, batch, Hkv, G, GT, ks, st;
+  int window;  // < 0: compressed keys (rule above); >= 0: ordinary keys, position i sees j in [i - window, i]
   long long qsn, qsh, ksn, ksh, vsn, vsh, osn, osh, dsn, dsh, dqsn, dqsh;
   float qk_scale, sm_scale;
 };
@@ -45,6 +46,17 @@ __device__ __forceinline__ int visible_keys(int pos, int lq, int lk, int ks, int
   if (pos >= lq || pos < ks - 1) return 0;
   const int n = (pos - ks + 1) / st + 1;
   return n < lk ? n : lk;
+}
+
+// half-open range [lo, hi) of keys visible to position pos
+__device__ __forceinline__ void visible_range(int pos, int lq, int lk, int ks, int st, int window, int& lo, int& hi) {
+  if (window < 0) {
+    lo = 0;
+    hi = visible_keys(pos, lq, lk, ks, st);
+  } else {
+    hi = pos < lq ? min(pos + 1, lk) : 0;
+    lo = hi > 0 ? max(0, pos - window) : 0;
+  }
 }
 
 // stage rows [32*chunk, +32) of up to two [*, H, D] tensors into LDS tiles (zeros past lk)
@@ -109,20 +121,24 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   const bool has_head = hq < p.G;
   const int hh = h * p.G + (has_head ? hq : 0);
   v8 qf[4][NK];
-  int lim[4];
-  int wave_lim = 0;
+  int lo[4], hi[4];
+  int wave_lo = 1 << 30, wave_hi = 0;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     const int pos = ti.i0 + 4 * wave + j;
-    lim[j] = visible_keys(pos, ti.lq, ti.lk, p.ks, p.st);
-    wave_lim = max(wave_lim, lim[j]);
+    visible_range(pos, ti.lq, ti.lk, p.ks, p.st, p.window, lo[j], hi[j]);
+    wave_hi = max(wave_hi, hi[j]);
+    if (hi[j] > 0) wave_lo = min(wave_lo, lo[j]);
     const bool live = has_head && pos < ti.lq;
     const T* qp = (const T*)p.q + (long long)(ti.s0q + (pos < ti.lq ? pos : 0)) * p.qsn + (long long)hh * p.qsh + 8 * lg;
 #pragma unroll
     for (int kk = 0; kk < NK; kk++) qf[j][kk] = live ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
   }
-  const int tile_last = min(ti.i0 + 15, ti.lq - 1);
-  const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
+  int tile_lo, tile_hi, unused;
+  visible_range(min(ti.i0 + 15, ti.lq - 1), ti.lq, ti.lk, p.ks, p.st, p.window, unused, tile_hi);
+  visible_range(ti.i0, ti.lq, ti.lk, p.ks, p.st, p.window, tile_lo, unused);
+  const int ch0 = tile_lo / 32;                 // the first token of the tile reaches furthest back
+  const int n_chunks = (tile_hi + 31) / 32;
   f32x4 acc[4][NDT];
   float m[4], l[4];
 #pragma unroll
@@ -134,15 +150,15 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
   const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
   Stager<T, D, 2> stg;
-  if (n_chunks > 0) {
-    stg.fetch(kb, p.ksn, vb, p.vsn, 0, ti.lk, tid);
+  if (n_chunks > ch0) {
+    stg.fetch(kb, p.ksn, vb, p.vsn, ch0, ti.lk, tid);
     stg.stash(k_s[0], v_s[0], tid);
   }
   __syncthreads();
-  for (int ch = 0; ch < n_chunks; ch++) {
-    const int buf = ch & 1;
+  for (int ch = ch0; ch < n_chunks; ch++) {
+    const int buf = (ch - ch0) & 1;
     if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, vb, p.vsn, ch + 1, ti.lk, tid);
-    if (32 * ch < wave_lim) {
+    if (32 * ch < wave_hi && 32 * ch + 32 > wave_lo) {
       f32x4 s[4][2];
 #pragma unroll
       for (int sub = 0; sub < 2; sub++) {
@@ -166,7 +182,7 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             const int c = 32 * ch + 16 * sub + 4 * lg + r;
-            const float x = c < lim[j] ? s[j][sub][r] * p.qk_scale : -INFINITY;
+            const float x = (c >= lo[j] && c < hi[j]) ? s[j][sub][r] * p.qk_scale : -INFINITY;
             s[j][sub][r] = x;
             mloc = fmaxf(mloc, x);
           }
@@ -598,7 +614,7 @@ static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, c
   p.q = q; p.k = k; p.v = v; p.cu_q = cu_q; p.cu_k = cu_k; p.total_q = (int)Tq; p.batch = (int)B; p.Hkv = (int)Hkv;
   p.G = (int)(Hq / Hkv); p.GT = (p.G + 15) / 16; p.ks = (int)ks; p.st = (int)st;
   p.qsn = strides[0]; p.qsh = strides[1]; p.ksn = strides[2]; p.ksh = strides[3]; p.vsn = strides[4]; p.vsh = strides[5];
-  p.qk_scale = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale;
+  p.qk_scale = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale; p.window = -1;
   p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr;
   a.Tq = Tq; a.Tk = Tk; a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.stream = (hipStream_t)stream; a.ws = nullptr;
   return NSA_OK;
@@ -666,5 +682,20 @@ extern "C" int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, con
   a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
   a.ws = (char*)workspace;
   a.what = 2;
+  return cmp_dispatch(a, head_dim, dtype);
+}
+
+// Causal sliding-window (or, with a window >= the longest sequence, plain causal) varlen attention,
+// forward only: the same tile kernel with the visibility rule "j in [i - window, i]".
+extern "C" int nsa_window_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
+                                   int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                   int64_t window_size, const int64_t* strides, float sm_scale, int dtype, void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, v, cu_seqlens, cu_seqlens, total_len, total_len, batch, num_q_heads, num_kv_heads, 1, 1, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!v || !o || !lse || window_size < 0 || strides[6] % 4 != 0 || strides[7] % 4 != 0 || (uintptr_t)o % 8 != 0) return NSA_ERR_BAD_ARG;
+  a.p.o = o; a.p.lse = lse; a.p.osn = strides[6]; a.p.osh = strides[7];
+  a.p.window = (int)(window_size > (1 << 30) ? (1 << 30) : window_size);
+  a.what = 0;
   return cmp_dispatch(a, head_dim, dtype);
 }

@@ -1,0 +1,109 @@
+"""Prefill / decode orchestration of the three NSA branches over an NSACache.
+
+Counterpart of the reference's nsa_infer (native_sparse_attention/infer/nsa_inference.py:24-151) and of
+the per-branch helpers in infer/inference_func.py:27-202, with the same argument order and
+conventions: step == 0 is the prefill over varlen tensors, step > 0 decodes one token per
+sequence; ``cu_seqlens`` always describes the prompt, so the cache holds prompt_len + step tokens
+after the update; ``rope(x, cu_seqlens, step, stride=1)`` is supplied by the caller.
+"""
+from typing import Callable, Optional, Tuple
+
+import torch
+
+from ..ops import (
+    compressed_attention,
+    compressed_attention_decode,
+    flash_attention_decode,
+    topk_sparse_attention,
+    topk_sparse_attention_decode,
+)
+from ..ops.sliding_window import sliding_window_attention_varlen
+from ..ops.utils import get_compressed_seqlens
+
+
+def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, intra_block_pe, kernel_size, kernel_stride):
+    if step == 0:
+        key, compress_cu_seqlens = compress_func[0](key, weight[0], cu_seqlens, kernel_size, kernel_stride, intra_block_pe)
+        value, _ = compress_func[1](value, weight[1], cu_seqlens, kernel_size, kernel_stride)
+        return key, value, compress_cu_seqlens
+    # decode: compress every sequence's staging window -> exactly one candidate token per sequence
+    batch = cu_seqlens.shape[0] - 1
+    aux_cu = torch.arange(batch + 1, dtype=torch.int32, device=cu_seqlens.device) * kernel_size
+    stage = cache.before_compress_kv_cache[:, :batch].reshape(2, batch * kernel_size, cache.num_kv_heads, cache.head_dim)
+    key, _ = compress_func[0](stage[0], weight[0], aux_cu, kernel_size, kernel_stride, intra_block_pe)
+    value, _ = compress_func[1](stage[1], weight[1], aux_cu, kernel_size, kernel_stride)
+    compress_cu_seqlens = torch.zeros(batch + 1, dtype=torch.int32, device=key.device)
+    compress_cu_seqlens[1:] = torch.cumsum(cache.compress_kv_len[:batch], dim=0)  # lengths before this token
+    return key, value, compress_cu_seqlens
+
+
+def compressed_attention_infer(cu_seqlens, step, query, key, value, cache, kernel_size, kernel_stride, topk, block_size,
+                               init_blocks, local_blocks):
+    if step == 0:
+        seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
+        comp_seqlens, comp_cu = get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)
+        return compressed_attention(query, key, value, kernel_size, kernel_stride, block_size, topk, cu_seqlens, comp_cu,
+                                    int(seqlens.max()), int(comp_seqlens.max()), None, init_blocks, local_blocks)
+    batch = cu_seqlens.shape[0] - 1
+    seqlens = cu_seqlens[1:] - cu_seqlens[:-1] + step
+    rows = int(cache.compress_kv_len[:batch].max())
+    return compressed_attention_decode(query, cache.compress_kv_cache[0, :batch, :rows], cache.compress_kv_cache[1, :batch, :rows],
+                                       seqlens, cache.compress_kv_len[:batch], kernel_size, kernel_stride, block_size, topk,
+                                       init_blocks, local_blocks)
+
+
+def topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size):
+    if step == 0:
+        return topk_sparse_attention(query, key, value, topk_idx, block_size, cu_seqlens)
+    batch = cu_seqlens.shape[0] - 1
+    return topk_sparse_attention_decode(query, cache.sparse_kv_cache[0, :batch], cache.sparse_kv_cache[1, :batch], topk_idx,
+                                        block_size, cache.sparse_kv_len[:batch])
+
+
+def sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size):
+    if step == 0:
+        return sliding_window_attention_varlen(query, key, value, cu_seqlens, window_size)
+    batch = cu_seqlens.shape[0] - 1
+    lens = torch.clamp(cache.sliding_kv_len[:batch], max=window_size)
+    return flash_attention_decode(query, cache.sliding_kv_cache[0, :batch], cache.sliding_kv_cache[1, :batch], lens)
+
+
+def nsa_infer(
+    cu_seqlens: torch.Tensor,
+    step: int,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    gate_value: torch.Tensor,
+    rope,
+    cache,
+    compress_weight: Tuple[torch.Tensor, torch.Tensor],
+    compress_func: Tuple[Callable, Callable],
+    intra_block_pe: Optional[torch.Tensor],
+    kernel_size: int,
+    kernel_stride: int,
+    block_size: int,
+    topk: int,
+    init_blocks: int,
+    local_blocks: int,
+    window_size: int,
+    return_branches: bool = False,
+) -> torch.Tensor:
+    """Gated sum of the compressed, selected and sliding-window branches; same shape as ``query``."""
+    if step == 0:
+        cache.reset()
+    cache.prepare_compress(cu_seqlens, step, key, value)
+    compress_key, compress_value, compress_cu = compress_infer(
+        cu_seqlens, step, key, value, cache, compress_weight, compress_func, intra_block_pe, kernel_size, kernel_stride)
+    query = rope(query, cu_seqlens, step)
+    compress_key = rope(compress_key, compress_cu, step if step == 0 else 1, stride=cache.kernel_stride)
+    key = rope(key, cu_seqlens, step)
+    cache.update_kv(cu_seqlens, step, compress_key, compress_value, key, value, key, value)
+    cmp_out, topk_idx = compressed_attention_infer(cu_seqlens, step, query, compress_key, compress_value, cache, kernel_size,
+                                                   kernel_stride, topk, block_size, init_blocks, local_blocks)
+    sparse_out = topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size)
+    window_out = sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size)
+    out = gate_value[..., 0, None] * cmp_out + gate_value[..., 1, None] * sparse_out + gate_value[..., 2, None] * window_out
+    if return_branches:
+        return out, (cmp_out, sparse_out, window_out, topk_idx)
+    return out

