@@ -59,23 +59,26 @@ __device__ __forceinline__ void visible_range(int pos, int lq, int lk, int ks, i
   }
 }
 
-// stage rows [32*chunk, +32) of up to two [*, H, D] tensors into LDS tiles (zeros past lk)
+// stage rows [32*chunk, +32) of one or two [*, H, D] tensors into LDS tiles (zeros past lk).  The two
+// tensors are handled by separate unrolled loops (no run-time choice of the base pointer).
 template <typename T, int D, int NTENS>
 struct Stager {
-  static constexpr int PIECES = NTENS * 32 * (D / 8);
+  static constexpr int PIECES = 32 * (D / 8);  // per tensor
   static constexpr int PPT = (PIECES + 255) / 256;
-  uint4 regs[PPT];
+  uint4 ra[PPT], rb[PPT];
+  unsigned ok;
+  // branch-free: always load (from a clamped row), mask when writing to LDS
   __device__ __forceinline__ void fetch(const T* a, long long asn, const T* b2, long long bsn, int chunk, int lk, int tid) {
+    ok = 0;
 #pragma unroll
     for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * 256;
-      uint4 val = {0u, 0u, 0u, 0u};
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), r = (pc / (D / 8)) % 32, which = pc / (D / 8) / 32;
-        const int key = chunk * 32 + r;
-        if (key < lk) val = *reinterpret_cast<const uint4*>((which == 0 ? a + (long long)key * asn : b2 + (long long)key * bsn) + 8 * c);
-      }
-      regs[u] = val;
+      const int pc = min(tid + u * 256, PIECES - 1);
+      const int c = pc % (D / 8), r = pc / (D / 8);
+      const int key = chunk * 32 + r;
+      const int kc = min(key, lk - 1);
+      ra[u] = *reinterpret_cast<const uint4*>(a + (long long)kc * asn + 8 * c);
+      if (NTENS == 2) rb[u] = *reinterpret_cast<const uint4*>(b2 + (long long)kc * bsn + 8 * c);
+      ok |= (unsigned)(key < lk) << u;
     }
   }
   __device__ __forceinline__ void stash(T (*ta)[D + 8], T (*tb)[D + 8], int tid) {
@@ -83,8 +86,16 @@ struct Stager {
     for (int u = 0; u < PPT; u++) {
       const int pc = tid + u * 256;
       if (pc < PIECES) {
-        const int c = pc % (D / 8), r = (pc / (D / 8)) % 32, which = pc / (D / 8) / 32;
-        *reinterpret_cast<uint4*>(which == 0 ? &ta[r][8 * c] : &tb[r][8 * c]) = regs[u];
+        const int c = pc % (D / 8), r = pc / (D / 8);
+        const unsigned m = 0u - ((ok >> u) & 1u);  // all ones when the row exists
+        uint4 x = ra[u];
+        x.x &= m; x.y &= m; x.z &= m; x.w &= m;
+        *reinterpret_cast<uint4*>(&ta[r][8 * c]) = x;
+        if (NTENS == 2) {
+          uint4 y = rb[u];
+          y.x &= m; y.y &= m; y.z &= m; y.w &= m;
+          *reinterpret_cast<uint4*>(&tb[r][8 * c]) = y;
+        }
       }
     }
   }

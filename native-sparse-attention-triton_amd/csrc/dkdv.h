@@ -50,7 +50,7 @@ struct DkdvParams {
 };
 
 template <typename T, int D, int BS, bool RANGE>
-__global__ __launch_bounds__(BS >= 64 ? 256 : 128) void dkdv_kernel(DkdvParams p) {
+__global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_kernel(DkdvParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16;
@@ -103,72 +103,80 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128) void dkdv_kernel(DkdvParams p
 #pragma unroll
     for (int i = 0; i < NDT; i++) { dk[j][i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[j][i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
-  // staging: 2 row groups x 16 heads x D elements for each of Q and dO = 2*2*16*D/8 16-byte pieces
-  constexpr int PIECES = 2 * 2 * 16 * (D / 8);
+  // staging: 2 row groups x 16 heads x D elements of Q and of dO per step, as 16-byte pieces.
+  // Q and dO are handled by separate, fully unrolled loops: selecting the tensor at run time makes
+  // the compiler fetch base pointers from a table and serialises the prefetch behind those loads.
+  constexpr int PIECES = 2 * 16 * (D / 8);       // per tensor
   constexpr int PPT = (PIECES + NT - 1) / NT;
-  uint4 stage[PPT];
-  float st_lse = 0.f, st_delta = 0.f;
-  int st_pos = 0;
-
-  auto fetch = [&](int step) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * NT;
-      uint4 val = {0u, 0u, 0u, 0u};
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = (pc / (D / 8) / 16) % 2, which = pc / (D / 8) / 32;
-        const int r = step * 2 + rg;
-        if (r < n_rg) {
-          const int t = RANGE ? first + r / p.GT : p.queries[first + r / p.GT];
-          const int hq = (r % p.GT) * 16 + hd;
-          if (hq < p.G) {
-            const T* src = which == 0 ? (const T*)p.q + (long long)t * p.qsn + (long long)(h * p.G + hq) * p.qsh
-                                      : (const T*)p.dout + (long long)t * p.dsn + (long long)(h * p.G + hq) * p.dsh;
-            val = *reinterpret_cast<const uint4*>(src + 8 * c);
-          }
-        }
-      }
-      stage[u] = val;
-    }
-    if (tid < 32) {
-      const int rg = tid >> 4, hd = tid & 15;
-      const int r = step * 2 + rg;
-      st_lse = INFINITY; st_delta = 0.f; st_pos = -1;
-      if (r < n_rg) {
-        const int t = RANGE ? first + r / p.GT : p.queries[first + r / p.GT];
-        const int hq = (r % p.GT) * 16 + hd;
-        st_pos = t - s0;
-        if (hq < p.G) {
-          st_lse = p.lse[(long long)(h * p.G + hq) * p.total_len + t];
-          st_delta = p.delta[(long long)(h * p.G + hq) * p.total_len + t];
-        }
-      }
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * NT;
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = (pc / (D / 8) / 16) % 2, which = pc / (D / 8) / 32;
-        T* dst = which == 0 ? &q_s[buf][rg][hd][8 * c] : &do_s[buf][rg][hd][8 * c];
-        *reinterpret_cast<uint4*>(dst) = stage[u];
-      }
-    }
-    if (tid < 32) {
-      lse_s[buf][tid] = st_lse;
-      delta_s[buf][tid] = st_delta;
-      if ((tid & 15) == 0) pos_s[buf][tid >> 4] = st_pos;
-    }
-  };
-
-  fetch(0);
-  stash(0);
+  // token ids of this chunk, read once (list mode); every later global load then has a single
+  // level of dependence and can be issued two steps ahead
+  __shared__ int tok_s[CHUNK_TOKENS];
+  for (int i = tid; i < n_tok; i += NT) tok_s[i] = RANGE ? first + i : p.queries[first + i];
   __syncthreads();
-  for (int step = 0; step < n_step; step++) {
-    const int buf = step & 1;
-    if (step + 1 < n_step) fetch(step + 1);
+  // fetch() is branch-free: loads are always issued (from a clamped, valid address) and the
+  // validity mask is applied when the registers are written to LDS.  Conditional loads make the
+  // compiler wait for every outstanding load at each join, which defeats the prefetch.
+  struct Stage { uint4 qd[PPT]; uint4 dd[PPT]; float lse, delta; int pos; unsigned ok; };
+  Stage stg[2];
+  const T* const qbase = (const T*)p.q + (long long)h * p.G * p.qsh;
+  const T* const dbase = (const T*)p.dout + (long long)h * p.G * p.dsh;
+  const float* const lbase = p.lse + (long long)h * p.G * p.total_len;
+  const float* const ebase = p.delta + (long long)h * p.G * p.total_len;
 
+  auto fetch = [&](int step, Stage& sg) {
+    unsigned ok = 0;
+#pragma unroll
+    for (int u = 0; u < PPT; u++) {
+      const int pc = min(tid + u * NT, PIECES - 1);
+      const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = pc / (D / 8) / 16;
+      const int r = step * 2 + rg;
+      const int rc = min(r, n_rg - 1);
+      const int t = tok_s[rc / p.GT];
+      const int hq = (rc % p.GT) * 16 + hd;
+      const int hc = min(hq, p.G - 1);
+      sg.qd[u] = *reinterpret_cast<const uint4*>(qbase + (long long)t * p.qsn + (long long)hc * p.qsh + 8 * c);
+      sg.dd[u] = *reinterpret_cast<const uint4*>(dbase + (long long)t * p.dsn + (long long)hc * p.dsh + 8 * c);
+      ok |= (unsigned)(r < n_rg && hq < p.G) << u;
+    }
+    {
+      const int rg = (tid >> 4) & 1, hd = tid & 15;
+      const int r = step * 2 + rg;
+      const int rc = min(r, n_rg - 1);
+      const int t = tok_s[rc / p.GT];
+      const int hq = (rc % p.GT) * 16 + hd;
+      const int hc = min(hq, p.G - 1);
+      sg.lse = lbase[(long long)hc * p.total_len + t];
+      sg.delta = ebase[(long long)hc * p.total_len + t];
+      sg.pos = r < n_rg ? t - s0 : -1;
+      ok |= (unsigned)(r < n_rg && hq < p.G) << 31;
+    }
+    sg.ok = ok;
+  };
+  auto stash = [&](int buf, const Stage& sg) {
+#pragma unroll
+    for (int u = 0; u < PPT; u++) {
+      const int pc = tid + u * NT;
+      if (pc < PIECES) {
+        const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = pc / (D / 8) / 16;
+        const unsigned m = 0u - ((sg.ok >> u) & 1u);  // all ones when the piece exists
+        uint4 a = sg.qd[u], b2 = sg.dd[u];
+        a.x &= m; a.y &= m; a.z &= m; a.w &= m;
+        b2.x &= m; b2.y &= m; b2.z &= m; b2.w &= m;
+        *reinterpret_cast<uint4*>(&q_s[buf][rg][hd][8 * c]) = a;
+        *reinterpret_cast<uint4*>(&do_s[buf][rg][hd][8 * c]) = b2;
+      }
+    }
+    if (tid < 32) {
+      const bool ok = sg.ok >> 31;
+      lse_s[buf][tid] = ok ? sg.lse : INFINITY;   // +inf -> probability 0 for rows that do not exist
+      delta_s[buf][tid] = ok ? sg.delta : 0.f;
+      if ((tid & 15) == 0) pos_s[buf][tid >> 4] = sg.pos;
+    }
+  };
+
+  // one step of the pipeline with compile-time buffer / register-set roles (no run-time choice of
+  // the register set, which would force copies that wait for the loads in flight)
+  auto compute = [&](const int buf) {
     // S = Q K^T and dP = dO V^T for this wave's keys; lane holds column key=li, rows 4*lg+r of each token
     v8 pf[KT], dsf[KT];
 #pragma unroll
@@ -220,8 +228,21 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128) void dkdv_kernel(DkdvParams p
         dk[j][dt] = E::mfma16(qtf, dsf[j], dk[j][dt]);
       }
     }
-    if (step + 1 < n_step) stash(buf ^ 1);
+  };
+  auto pipeline_step = [&](int step, const int buf, Stage& refill, const Stage& ready) {
+    // `refill` was written to LDS one step ago: reuse it for step + 2 (clamped: the tail re-loads the last step)
+    fetch(min(step + 2, n_step - 1), refill);
+    compute(buf);
+    if (step + 1 < n_step) stash(buf ^ 1, ready);
     __syncthreads();
+  };
+  fetch(0, stg[0]);
+  stash(0, stg[0]);
+  fetch(min(1, n_step - 1), stg[1]);
+  __syncthreads();
+  for (int step = 0; step < n_step; step += 2) {
+    pipeline_step(step, 0, stg[0], stg[1]);
+    if (step + 1 < n_step) pipeline_step(step + 1, 1, stg[1], stg[0]);
   }
   // partial[item][0 = dK, 1 = dV][key][d], fp32
   float* out = p.partial + (long long)item * 2 * BS * D;

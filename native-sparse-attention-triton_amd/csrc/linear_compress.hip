@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void lin_dw_kernel(LinParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NET = D / 16, LD = D + 8, PIECES = 2 * 32 * (D / 8), PPT = (PIECES + 255) / 256;
+  constexpr int NET = D / 16, LD = D + 8;
   constexpr int DTW = (D / 16 + 3) / 4;  // d tiles per wave
   __shared__ __attribute__((aligned(16))) T x_s[2][32][LD];
   __shared__ __attribute__((aligned(16))) T g_s[2][32][LD];
@@ -173,35 +173,33 @@ __global__ __launch_bounds__(256) void lin_dw_kernel(LinParams p) {
   for (int a = 0; a < DTW; a++)
 #pragma unroll
     for (int i = 0; i < NET; i++) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  uint4 regs[PPT];
+  constexpr int PIECES1 = 32 * (D / 8), PPT1 = (PIECES1 + 255) / 256;  // per tensor
+  uint4 rx[PPT1], rg[PPT1];
   auto fetch = [&](int chunk) {
 #pragma unroll
-    for (int u = 0; u < PPT; u++) {
+    for (int u = 0; u < PPT1; u++) {
       const int pc = tid + u * 256;
-      uint4 val = {0u, 0u, 0u, 0u};
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), r = (pc / (D / 8)) % 32, which = pc / (D / 8) / 32;
-        const int n = chunk * 32 + r;
-        if (n < p.total_y) {
-          if (which == 0) {
-            const int b = find_sequence(p.ycu, p.batch, n);
-            const long long row = p.cu[b] + (long long)(n - p.ycu[b]) * p.st + k;
-            val = *reinterpret_cast<const uint4*>((const T*)p.x + row * p.xsn + (long long)h * p.xsh + 8 * c);
-          } else {
-            val = *reinterpret_cast<const uint4*>((const T*)p.dy + (long long)n * p.dysn + (long long)h * p.dysh + 8 * c);
-          }
-        }
+      const int c = pc % (D / 8), r = pc / (D / 8);
+      const int n = chunk * 32 + r;
+      uint4 vx = {0u, 0u, 0u, 0u}, vg = {0u, 0u, 0u, 0u};
+      if (pc < PIECES1 && n < p.total_y) {
+        const int b = find_sequence(p.ycu, p.batch, n);
+        const long long row = p.cu[b] + (long long)(n - p.ycu[b]) * p.st + k;
+        vx = *reinterpret_cast<const uint4*>((const T*)p.x + row * p.xsn + (long long)h * p.xsh + 8 * c);
+        vg = *reinterpret_cast<const uint4*>((const T*)p.dy + (long long)n * p.dysn + (long long)h * p.dysh + 8 * c);
       }
-      regs[u] = val;
+      rx[u] = vx;
+      rg[u] = vg;
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int u = 0; u < PPT; u++) {
+    for (int u = 0; u < PPT1; u++) {
       const int pc = tid + u * 256;
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), r = (pc / (D / 8)) % 32, which = pc / (D / 8) / 32;
-        *reinterpret_cast<uint4*>(which == 0 ? &x_s[buf][r][8 * c] : &g_s[buf][r][8 * c]) = regs[u];
+      if (pc < PIECES1) {
+        const int c = pc % (D / 8), r = pc / (D / 8);
+        *reinterpret_cast<uint4*>(&x_s[buf][r][8 * c]) = rx[u];
+        *reinterpret_cast<uint4*>(&g_s[buf][r][8 * c]) = rg[u];
       }
     }
   };
