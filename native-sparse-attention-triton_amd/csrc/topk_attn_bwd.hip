@@ -8,8 +8,8 @@
 //   3. dK/dV: a workgroup keeps one KV block's K and V rows in registers (each wave owns 16
 //      keys) and streams the queries of that block two tokens at a time through LDS; per-chunk
 //      fp32 partials are reduced in a fixed order, so the result is deterministic (no atomics).
-//   4. dQ: one wavefront per (token, kv-head), same dataflow as the forward kernel, with a
-//      block-transposed copy of K feeding dQ^T += K^T * dS^T.
+//   4. dQ: one wavefront per (token, kv-head), same dataflow as the forward kernel; the K rows are
+//      written through to wave-private LDS and read back transposed for dQ^T += K^T * dS^T.
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -21,9 +21,9 @@
 // ------------------------------------------------------------------------------------------
 // workspace carving (host and entry point must agree)
 struct BwdLayout {
-  size_t delta, cu_blk, keys_in, keys_out, vals_in, vals_out, seg_off, chunk_off, sort_tmp, kt, partial, total;
+  size_t delta, cu_blk, keys_in, keys_out, vals_in, vals_out, seg_off, chunk_off, sort_tmp, partial, total;
   size_t sort_tmp_bytes;
-  int64_t max_blocks, n_pairs, max_items, n_slots;
+  int64_t max_blocks, n_pairs, max_items;
 };
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -34,7 +34,6 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.n_pairs = Hkv * T * topk;
   const int64_t GT = (Hq / Hkv + 15) / 16;
   L.max_items = (L.n_pairs + CHUNK_TOKENS - 1) / CHUNK_TOKENS + Hkv * L.max_blocks;
-  L.n_slots = nsa_chunk_slots(T, B);
   (void)GT;
   size_t tmp = 0;
   uint32_t* nk = nullptr;
@@ -52,7 +51,6 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.seg_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.chunk_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.sort_tmp = take(tmp);
-  L.kt = take((size_t)Hkv * L.n_slots * D * 32 * 2);
   L.partial = take((size_t)L.max_items * bs * D * 4 * 2);
   L.total = off;
   return L;
@@ -105,9 +103,9 @@ __global__ __launch_bounds__(256) void segment_offsets_kernel(const uint32_t* __
 // ------------------------------------------------------------------------------------------
 // pass 4: dQ
 struct DqParams {
-  const void* q; const void* k; const void* v; const void* kt; const void* dout; const float* lse; const float* delta;
+  const void* q; const void* k; const void* v; const void* dout; const float* lse; const float* delta;
   const int32_t* idx; const int32_t* cu; void* dq;
-  int total_len, batch, Hkv, G, GT, topk, n_slots;
+  int total_len, batch, Hkv, G, GT, topk;
   long long n_items;
   long long qsn, qsh, ksn, ksh, vsn, vsh, dsn, dsh, ish, isn, isk, dqsn, dqsh;
   float qk_scale, sm_scale;
@@ -118,7 +116,13 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16, NCH = BS / 32;
+  constexpr int NK = D / 32, NDT = D / 16, NCH = BS / 32, LD = D + 8;
+  // wave-private staging of one 64-key slice of K: the rows arrive from global memory in A-operand
+  // layout for S^T = K Q^T, are written through to LDS, and come back transposed (K^T fragments)
+  // for dQ^T += K^T dS^T - K is fetched once per (token, block) instead of twice
+  __shared__ __attribute__((aligned(16))) T k_s[4][64][LD];
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
   const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
@@ -129,7 +133,6 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   const int b = find_sequence(p.cu, p.batch, t);
   const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
   const int pos = t - s0, qb = pos / BS;
-  const int slot0 = seq_first_slot(p.cu, b);
   const int hq = gt * 16 + li;
   const bool has_head = hq < p.G;
   const int hh = h * p.G + (has_head ? hq : 0);
@@ -149,42 +152,61 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   const int32_t* ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
   const T* kbase = (const T*)p.k + (long long)s0 * p.ksn + (long long)h * p.ksh + 8 * lg;
   const T* vbase = (const T*)p.v + (long long)s0 * p.vsn + (long long)h * p.vsh + 8 * lg;
-  const T* ktbase = (const T*)p.kt + ((long long)h * p.n_slots + slot0) * D * 32 + li * 32 + 8 * lg;
+  T (*ks)[LD] = k_s[wave];
+  // rows that a partly causal slice never stages are multiplied by dS = 0: they must hold finite values
+  for (int i = lane; i < 64 * LD / 8; i += 64) st16(&ks[0][0] + 8 * i, zero16<v8>());
   for (int e = 0; e < p.topk; e++) {
     const int blk = ip[(long long)e * p.isk];
     if (blk < 0 || blk > qb) continue;
-    const int key0 = blk * BS;
-    f32x4 ds[NSUB];
+    // 64 keys at a time (larger blocks are walked in 64-key slices)
 #pragma unroll
-    for (int nt = 0; nt < NSUB; nt++) {
-      f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-      if (key0 + 16 * nt <= pos) {
-        int row = key0 + 16 * nt + li;
-        row = row < len ? row : len - 1;
-        const T* kp = kbase + (long long)row * p.ksn;
-        const T* vp = vbase + (long long)row * p.vsn;
+    for (int half = 0; half < (BS + 63) / 64; half++) {
+      const int key0 = blk * BS + 64 * half;
+      if (key0 > pos) break;
+      constexpr int NS = BS >= 64 ? 4 : BS / 16;  // 16-key sub-tiles in this slice
+      f32x4 ds[NS];
 #pragma unroll
-        for (int kk = 0; kk < NK; kk++) {
-          s = E::mfma16(ld16<v8>(kp + 32 * kk), qf[kk], s);
-          dp = E::mfma16(ld16<v8>(vp + 32 * kk), dof[kk], dp);
+      for (int nt = 0; nt < NS; nt++) {
+        f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+        if (key0 + 16 * nt <= pos) {
+          int row = key0 + 16 * nt + li;
+          row = row < len ? row : len - 1;
+          const T* kp = kbase + (long long)row * p.ksn;
+          const T* vp = vbase + (long long)row * p.vsn;
+#pragma unroll
+          for (int kk = 0; kk < NK; kk++) {
+            const v8 kf = ld16<v8>(kp + 32 * kk);
+            st16(&ks[16 * nt + li][32 * kk + 8 * lg], kf);
+            s = E::mfma16(kf, qf[kk], s);
+            dp = E::mfma16(ld16<v8>(vp + 32 * kk), dof[kk], dp);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int key = key0 + 16 * nt + 4 * lg + r;
+          const float pr = key <= pos ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
+          ds[nt][r] = pr * (dp[r] - dl) * p.sm_scale;
         }
       }
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int key = key0 + 16 * nt + 4 * lg + r;
-        const float pr = key <= pos ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
-        ds[nt][r] = pr * (dp[r] - dl) * p.sm_scale;
+      for (int c = 0; c < (NS + 1) / 2; c++) {
+        if (key0 + 32 * c > pos) break;  // rows of a wholly masked chunk were never staged
+        v8 dsf;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          dsf[r] = (T)ds[2 * c][r];
+          dsf[4 + r] = (T)(2 * c + 1 < NS ? ds[(2 * c + 1) % NS][r] : 0.f);
+        }
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) {
+          const T* a0 = &ks[32 * c + 4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+          const T* a1 = &ks[32 * c + 16 + 4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+          s16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+          s16x4 y = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a1));
+          s16x8 z = {x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+          acc[dt] = E::mfma16(__builtin_bit_cast(v8, z), dsf, acc[dt]);
+        }
       }
-    }
-#pragma unroll
-    for (int c = 0; c < NCH; c++) {
-      if (key0 + 32 * c > pos) break;
-      v8 dsf;
-#pragma unroll
-      for (int r = 0; r < 4; r++) { dsf[r] = (T)ds[2 * c][r]; dsf[4 + r] = (T)ds[2 * c + 1][r]; }
-      const T* ktp = ktbase + (long long)((key0 >> 5) + c) * D * 32;
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++) acc[dt] = E::mfma16(ld16<v8>(ktp + dt * 16 * 32), dsf, acc[dt]);
     }
   }
   if (has_head) {
@@ -263,11 +285,9 @@ static int run_bwd(const BwdArgs& a) {
         p.partial, p.chunk_off, a.cu, p.cu_blk, (int)a.B, (int)L.max_blocks, (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
   }
   if (a.phases & NSA_BWD_PHASE_DQ) {
-    T* kt = (T*)(ws + L.kt);
-    launch_block_transpose<T, D>((const T*)a.k, kt, a.cu, a.B, a.ksn, a.ksh, L.n_slots, a.Hkv, a.stream);
     DqParams p;
-    p.q = a.q; p.k = a.k; p.v = a.v; p.kt = kt; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
-    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk; p.n_slots = (int)L.n_slots;
+    p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
+    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk;
     p.n_items = (long long)a.T * GT * a.Hkv;
     p.qsn = a.qsn; p.qsh = a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = a.dsn; p.dsh = a.dsh;
     p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
