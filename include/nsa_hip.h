@@ -39,9 +39,9 @@ int nsa_version(void);
  * (native_sparse_attention/ops/triton/topk_sparse_attention.py:828-909).
  *   q,o [T,Hq,D]; k,v [T,Hkv,D]; topk_idx int32 [Hkv,T,topk] (entries <0 or beyond the
  *   query's own block are skipped); lse fp32 [Hq,T] in base-2 units (contiguous).
- * workspace holds a block-transposed copy of V: nsa_topk_attn_fwd_workspace_bytes().
+ * workspace holds fragment-major copies of K and V (2x their size): nsa_topk_attn_fwd_workspace_bytes().
  * phases: NSA_FWD_PHASE_ALL, or a subset when the caller re-uses the workspace of a previous
- * call with the same V (profiling a single kernel).
+ * call with the same K and V (profiling a single kernel).
  */
 #define NSA_FWD_PHASE_TRANSPOSE 1
 #define NSA_FWD_PHASE_ATTEND 2

@@ -14,16 +14,16 @@
 
 #include <rocprim/device/device_radix_sort.hpp>
 
-#include "block_transpose.h"
+#include "retile.h"
 #include "delta.h"
 #include "dkdv.h"
 
 // ------------------------------------------------------------------------------------------
 // workspace carving (host and entry point must agree)
 struct BwdLayout {
-  size_t delta, cu_blk, keys_in, keys_out, vals_in, vals_out, seg_off, chunk_off, sort_tmp, partial, total;
+  size_t delta, cu_blk, keys_in, keys_out, vals_in, vals_out, seg_off, chunk_off, sort_tmp, kf, vf, partial, total;
   size_t sort_tmp_bytes;
-  int64_t max_blocks, n_pairs, max_items;
+  int64_t max_blocks, n_pairs, max_items, n_slots;
 };
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -51,6 +51,9 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.seg_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.chunk_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.sort_tmp = take(tmp);
+  L.n_slots = nsa_chunk_slots(T, B);
+  L.kf = take(retile_bytes(T, B, Hkv, D));   // row-fragment copies of K and V for the dQ pass
+  L.vf = take(retile_bytes(T, B, Hkv, D));
   L.partial = take((size_t)L.max_items * bs * D * 4 * 2);
   L.total = off;
   return L;
@@ -103,11 +106,11 @@ __global__ __launch_bounds__(256) void segment_offsets_kernel(const uint32_t* __
 // ------------------------------------------------------------------------------------------
 // pass 4: dQ
 struct DqParams {
-  const void* q; const void* k; const void* v; const void* dout; const float* lse; const float* delta;
+  const void* q; const void* kf; const void* vf; const void* dout; const float* lse; const float* delta;
   const int32_t* idx; const int32_t* cu; void* dq;
-  int total_len, batch, Hkv, G, GT, topk;
+  int total_len, batch, Hkv, G, GT, topk, n_slots;
   long long n_items;
-  long long qsn, qsh, ksn, ksh, vsn, vsh, dsn, dsh, ish, isn, isk, dqsn, dqsh;
+  long long qsn, qsh, dsn, dsh, ish, isn, isk, dqsn, dqsh;
   float qk_scale, sm_scale;
 };
 
@@ -117,8 +120,9 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   constexpr int NK = D / 32, NDT = D / 16, NCH = BS / 32, LD = D + 8;
-  // wave-private staging of one 64-key slice of K: the rows arrive from global memory in A-operand
-  // layout for S^T = K Q^T, are written through to LDS, and come back transposed (K^T fragments)
+  // K and V come from their fragment-major copies (one coalesced 1 KiB load per operand fragment).
+  // Wave-private staging of one 64-key slice of K: the fragments arrive in A-operand layout for
+  // S^T = K Q^T, are written through to LDS as rows, and come back transposed (K^T fragments)
   // for dQ^T += K^T dS^T - K is fetched once per (token, block) instead of twice
   __shared__ __attribute__((aligned(16))) T k_s[4][64][LD];
   typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -131,8 +135,9 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   const int gt = (int)((item / p.total_len) % p.GT);
   const int h = (int)(item / ((long long)p.total_len * p.GT));
   const int b = find_sequence(p.cu, p.batch, t);
-  const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
+  const int s0 = p.cu[b];
   const int pos = t - s0, qb = pos / BS;
+  const int slot0 = seq_first_slot(p.cu, b);
   const int hq = gt * 16 + li;
   const bool has_head = hq < p.G;
   const int hh = h * p.G + (has_head ? hq : 0);
@@ -150,8 +155,8 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
 #pragma unroll
   for (int i = 0; i < NDT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
-  const T* kbase = (const T*)p.k + (long long)s0 * p.ksn + (long long)h * p.ksh + 8 * lg;
-  const T* vbase = (const T*)p.v + (long long)s0 * p.vsn + (long long)h * p.vsh + 8 * lg;
+  const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
+  const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
   T (*ks)[LD] = k_s[wave];
   // rows that a partly causal slice never stages are multiplied by dS = 0: they must hold finite values
   for (int i = lane; i < 64 * LD / 8; i += 64) st16(&ks[0][0] + 8 * i, zero16<v8>());
@@ -169,16 +174,13 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
       for (int nt = 0; nt < NS; nt++) {
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
         if (key0 + 16 * nt <= pos) {
-          int row = key0 + 16 * nt + li;
-          row = row < len ? row : len - 1;
-          const T* kp = kbase + (long long)row * p.ksn;
-          const T* vp = vbase + (long long)row * p.vsn;
+          const long long frag = (long long)(((key0 >> 4) + nt) * NK) * 512;
 #pragma unroll
           for (int kk = 0; kk < NK; kk++) {
-            const v8 kf = ld16<v8>(kp + 32 * kk);
+            const v8 kf = ld16<v8>(kbase + frag + kk * 512);
             st16(&ks[16 * nt + li][32 * kk + 8 * lg], kf);
             s = E::mfma16(kf, qf[kk], s);
-            dp = E::mfma16(ld16<v8>(vp + 32 * kk), dof[kk], dp);
+            dp = E::mfma16(ld16<v8>(vbase + frag + kk * 512), dof[kk], dp);
           }
         }
 #pragma unroll
@@ -286,10 +288,14 @@ static int run_bwd(const BwdArgs& a) {
   }
   if (a.phases & NSA_BWD_PHASE_DQ) {
     DqParams p;
-    p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
-    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk;
+    T* kf = (T*)(ws + L.kf);
+    T* vf = (T*)(ws + L.vf);
+    launch_retile<T, D, RETILE_ROWS>((const T*)a.k, kf, a.cu, a.B, a.ksn, a.ksh, L.n_slots, a.Hkv, a.stream);
+    launch_retile<T, D, RETILE_ROWS>((const T*)a.v, vf, a.cu, a.B, a.vsn, a.vsh, L.n_slots, a.Hkv, a.stream);
+    p.q = a.q; p.kf = kf; p.vf = vf; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
+    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk; p.n_slots = (int)L.n_slots;
     p.n_items = (long long)a.T * GT * a.Hkv;
-    p.qsn = a.qsn; p.qsh = a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = a.dsn; p.dsh = a.dsh;
+    p.qsn = a.qsn; p.qsh = a.qsh; p.dsn = a.dsn; p.dsh = a.dsh;
     p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
     long long n_wg = ((p.n_items + 3) / 4 + 7) / 8 * 8;

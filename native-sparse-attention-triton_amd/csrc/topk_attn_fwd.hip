@@ -4,17 +4,17 @@
 // group.  Scores are produced transposed, S^T[key][head] = K * Q^T, so that each lane ends
 // up holding values of a single head: the row maximum and sum become per-lane scalars plus
 // two cross-lane steps, and P^T is already in the B-operand layout of the next MFMA,
-// O^T[d][head] += V^T[d][key] * P^T[key][head].  K rows are read straight from global memory
-// in A-operand layout (16 bytes per lane); V comes from the block-transposed copy built by
-// block_transpose_kernel.  Nothing is staged in LDS: with one token per wave every K/V
-// element feeds exactly one MFMA, so there is no reuse for LDS to exploit.
-#include "block_transpose.h"
+// O^T[d][head] += V^T[d][key] * P^T[key][head].  K and V are read from fragment-major copies
+// (retile.h): every operand fragment is one coalesced 1 KiB load.  Nothing is staged in LDS:
+// with one token per wave every K/V element feeds exactly one MFMA, so there is no reuse for
+// LDS to exploit.
+#include "retile.h"
 
 struct TopkFwdParams {
-  const void* q; const void* k; const void* vt; const int32_t* idx; void* o; float* lse; const int32_t* cu;
+  const void* q; const void* kf; const void* vf; const int32_t* idx; void* o; float* lse; const int32_t* cu;
   int total_len, batch, Hkv, G, GT, topk, n_slots;
   long long n_items;
-  long long qsn, qsh, ksn, ksh, ish, isn, isk, osn, osh;
+  long long qsn, qsh, ish, isn, isk, osn, osh;
   float qk_scale;  // sm_scale * log2(e)
 };
 
@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
   const int gt = (int)((item / p.total_len) % p.GT);
   const int h = (int)(item / ((long long)p.total_len * p.GT));
   const int b = find_sequence(p.cu, p.batch, t);
-  const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
+  const int s0 = p.cu[b];
   const int pos = t - s0, qb = pos / BS;
   const int slot0 = seq_first_slot(p.cu, b);
 
@@ -49,8 +49,8 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
   float m = -INFINITY, lsum = 0.f;
 
   const int32_t* ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
-  const T* kbase = (const T*)p.k + (long long)s0 * p.ksn + (long long)h * p.ksh + 8 * lg;
-  const T* vbase = (const T*)p.vt + ((long long)h * p.n_slots + slot0) * D * 32 + li * 32 + 8 * lg;
+  const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
+  const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
 
   for (int e = 0; e < p.topk; e++) {
     const int blk = ip[(long long)e * p.isk];
@@ -59,13 +59,12 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
     f32x4 s[NSUB];
 #pragma unroll
     for (int nt = 0; nt < NSUB; nt++) {
-      int row = key0 + 16 * nt + li;
-      row = row < len ? row : len - 1;
-      const T* kp = kbase + (long long)row * p.ksn;
+      // fragment (slot, sub, kk) of the row-fragment copy: 512 elements each
+      const T* kp = kbase + (long long)(((key0 >> 4) + nt) * NK) * 512;
       f32x4 c = {0.f, 0.f, 0.f, 0.f};
       if (key0 + 16 * nt <= pos) {  // wave-uniform: sub-tiles wholly in the future are never loaded
 #pragma unroll
-        for (int kk = 0; kk < NK; kk++) c = E::mfma16(ld16<v8>(kp + 32 * kk), qf[kk], c);
+        for (int kk = 0; kk < NK; kk++) c = E::mfma16(ld16<v8>(kp + kk * 512), qf[kk], c);
       }
       s[nt] = c;
     }
@@ -107,7 +106,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
       }
       const T* vp = vbase + (long long)((key0 >> 5) + c) * D * 32;
 #pragma unroll
-      for (int dt = 0; dt < NDT; dt++) acc[dt] = E::mfma16(ld16<v8>(vp + dt * 16 * 32), pf, acc[dt]);
+      for (int dt = 0; dt < NDT; dt++) acc[dt] = E::mfma16(ld16<v8>(vp + dt * 512), pf, acc[dt]);
     }
   }
   lsum += __shfl_xor(lsum, 16);
@@ -127,9 +126,12 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
 }
 
 template <typename T, int D, int BS>
-static int launch_fwd(const TopkFwdParams& p, const void* v, long long vsn, long long vsh, int phases, hipStream_t stream) {
-  if (phases & NSA_FWD_PHASE_TRANSPOSE)
-    launch_block_transpose<T, D>((const T*)v, (T*)p.vt, p.cu, p.batch, vsn, vsh, p.n_slots, p.Hkv, stream);
+static int launch_fwd(const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn, long long vsh,
+                      int phases, hipStream_t stream) {
+  if (phases & NSA_FWD_PHASE_TRANSPOSE) {
+    launch_retile<T, D, RETILE_ROWS>((const T*)k, (T*)p.kf, p.cu, p.batch, ksn, ksh, p.n_slots, p.Hkv, stream);
+    launch_retile<T, D, RETILE_COLS>((const T*)v, (T*)p.vf, p.cu, p.batch, vsn, vsh, p.n_slots, p.Hkv, stream);
+  }
   if (phases & NSA_FWD_PHASE_ATTEND) {
     long long n_wg = (p.n_items + 3) / 4;
     n_wg = (n_wg + 7) / 8 * 8;
@@ -139,29 +141,31 @@ static int launch_fwd(const TopkFwdParams& p, const void* v, long long vsn, long
 }
 
 template <typename T, int D>
-static int dispatch_bs(int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, int ph, hipStream_t s) {
+static int dispatch_bs(int bs, const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn, long long vsh,
+                       int ph, hipStream_t s) {
   switch (bs) {
-    case 32: return launch_fwd<T, D, 32>(p, v, vsn, vsh, ph, s);
-    case 64: return launch_fwd<T, D, 64>(p, v, vsn, vsh, ph, s);
-    case 128: return launch_fwd<T, D, 128>(p, v, vsn, vsh, ph, s);
-    case 256: return launch_fwd<T, D, 256>(p, v, vsn, vsh, ph, s);
+    case 32: return launch_fwd<T, D, 32>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 64: return launch_fwd<T, D, 64>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 128: return launch_fwd<T, D, 128>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 256: return launch_fwd<T, D, 256>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
   }
   return NSA_ERR_UNSUPPORTED;
 }
 
 template <typename T>
-static int dispatch_d(int d, int bs, const TopkFwdParams& p, const void* v, long long vsn, long long vsh, int ph, hipStream_t s) {
+static int dispatch_d(int d, int bs, const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn,
+                      long long vsh, int ph, hipStream_t s) {
   switch (d) {
-    case 32: return dispatch_bs<T, 32>(bs, p, v, vsn, vsh, ph, s);
-    case 64: return dispatch_bs<T, 64>(bs, p, v, vsn, vsh, ph, s);
-    case 96: return dispatch_bs<T, 96>(bs, p, v, vsn, vsh, ph, s);
-    case 128: return dispatch_bs<T, 128>(bs, p, v, vsn, vsh, ph, s);
+    case 32: return dispatch_bs<T, 32>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 64: return dispatch_bs<T, 64>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 96: return dispatch_bs<T, 96>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 128: return dispatch_bs<T, 128>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
   }
   return NSA_ERR_UNSUPPORTED;
 }
 
 extern "C" size_t nsa_topk_attn_fwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t head_dim) {
-  return (size_t)num_kv_heads * (size_t)nsa_chunk_slots(total_len, batch) * (size_t)head_dim * 32 * 2;
+  return 2 * retile_bytes(total_len, batch, num_kv_heads, head_dim);  // K and V copies
 }
 
 extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t* topk_idx, void* o, float* lse,
@@ -180,16 +184,16 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)workspace) % 16 != 0 || (uintptr_t)o % 8 != 0) return NSA_ERR_UNSUPPORTED;
   if (workspace_bytes < nsa_topk_attn_fwd_workspace_bytes(total_len, batch, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
   TopkFwdParams p;
-  p.q = q; p.k = k; p.vt = workspace; p.idx = topk_idx; p.o = o; p.lse = lse; p.cu = cu_seqlens;
+  p.q = q; p.kf = workspace; p.vf = (char*)workspace + retile_bytes(total_len, batch, num_kv_heads, head_dim); p.idx = topk_idx; p.o = o; p.lse = lse; p.cu = cu_seqlens;
   p.total_len = (int)total_len; p.batch = (int)batch; p.Hkv = (int)num_kv_heads; p.G = (int)(num_q_heads / num_kv_heads);
   p.GT = (p.G + 15) / 16; p.topk = (int)topk; p.n_slots = (int)nsa_chunk_slots(total_len, batch);
   p.n_items = (long long)total_len * p.GT * p.Hkv;
-  p.qsn = q_stride_n; p.qsh = q_stride_h; p.ksn = k_stride_n; p.ksh = k_stride_h;
+  p.qsn = q_stride_n; p.qsh = q_stride_h;
   p.ish = idx_stride_h; p.isn = idx_stride_n; p.isk = idx_stride_k; p.osn = o_stride_n; p.osh = o_stride_h;
   p.qk_scale = sm_scale * NSA_LOG2E;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, phases, s);
-  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, v, v_stride_n, v_stride_h, phases, s);
+  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, k, k_stride_n, k_stride_h, v, v_stride_n, v_stride_h, phases, s);
+  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, k, k_stride_n, k_stride_h, v, v_stride_n, v_stride_h, phases, s);
   return NSA_ERR_UNSUPPORTED;
 }
 
