@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   const int gt = (int)((item / p.total_len) % p.GT);
   const int h = (int)(item / ((long long)p.total_len * p.GT));
   const int b = find_sequence(p.cu, p.batch, t);
-  const int s0 = p.cu[b];
+  const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
   const int pos = t - s0, qb = pos / BS;
   const int slot0 = seq_first_slot(p.cu, b);
   const int hq = gt * 16 + li;
@@ -158,30 +158,42 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
   const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
   T (*ks)[LD] = k_s[wave];
-  // rows that a partly causal slice never stages are multiplied by dS = 0: they must hold finite values
-  for (int i = lane; i < 64 * LD / 8; i += 64) st16(&ks[0][0] + 8 * i, zero16<v8>());
-  for (int e = 0; e < p.topk; e++) {
-    const int blk = ip[(long long)e * p.isk];
-    if (blk < 0 || blk > qb) continue;
-    // 64 keys at a time (larger blocks are walked in 64-key slices)
+  const int last_slot = (len - 1) >> 5;
+  // block ids are read once (lane e holds entry e) and visited through a wave-uniform bit mask
+  for (int e0 = 0; e0 < p.topk; e0 += 64) {
+  const int my_e = e0 + lane;
+  const int my_blk = my_e < p.topk ? ip[(long long)my_e * p.isk] : -1;
+  unsigned long long todo = __ballot(my_blk >= 0 && my_blk <= qb);
+  while (todo) {
+    const int e = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    const int blk = __builtin_amdgcn_readlane(my_blk, e);
+    // 64 keys at a time (larger blocks are walked in 64-key slices); all fragment loads of a slice
+    // are issued back to back before any of them is consumed
 #pragma unroll
     for (int half = 0; half < (BS + 63) / 64; half++) {
       const int key0 = blk * BS + 64 * half;
       if (key0 > pos) break;
       constexpr int NS = BS >= 64 ? 4 : BS / 16;  // 16-key sub-tiles in this slice
+      v8 kfr[NS][NK], vfr[NS][NK];
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++) {
+        const int st = min((key0 >> 4) + nt, 2 * last_slot + 1);  // future sub-tiles: clamp onto existing storage
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) {
+          kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512);
+          vfr[nt][kk] = ld16<v8>(vbase + (long long)(st * NK + kk) * 512);
+        }
+      }
       f32x4 ds[NS];
 #pragma unroll
       for (int nt = 0; nt < NS; nt++) {
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-        if (key0 + 16 * nt <= pos) {
-          const long long frag = (long long)(((key0 >> 4) + nt) * NK) * 512;
 #pragma unroll
-          for (int kk = 0; kk < NK; kk++) {
-            const v8 kf = ld16<v8>(kbase + frag + kk * 512);
-            st16(&ks[16 * nt + li][32 * kk + 8 * lg], kf);
-            s = E::mfma16(kf, qf[kk], s);
-            dp = E::mfma16(ld16<v8>(vbase + frag + kk * 512), dof[kk], dp);
-          }
+        for (int kk = 0; kk < NK; kk++) {
+          st16(&ks[16 * nt + li][32 * kk + 8 * lg], kfr[nt][kk]);
+          s = E::mfma16(kfr[nt][kk], qf[kk], s);
+          dp = E::mfma16(vfr[nt][kk], dof[kk], dp);
         }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -192,8 +204,7 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
       }
 #pragma unroll
       for (int c = 0; c < (NS + 1) / 2; c++) {
-        if (key0 + 32 * c > pos) break;  // rows of a wholly masked chunk were never staged
-        v8 dsf;
+        v8 dsf;  // dS of masked keys is exactly 0; the (clamped, finite) K rows it meets do not matter
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           dsf[r] = (T)ds[2 * c][r];
@@ -210,6 +221,7 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
         }
       }
     }
+  }
   }
   if (has_head) {
     T* op = (T*)p.dq + (long long)t * p.dqsn + (long long)hh * p.dqsh + 4 * lg;

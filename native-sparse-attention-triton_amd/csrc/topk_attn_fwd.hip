@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16, NCH = BS / 32;
+  constexpr int NK = D / 32, NDT = D / 16;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
   const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
   const int gt = (int)((item / p.total_len) % p.GT);
   const int h = (int)(item / ((long long)p.total_len * p.GT));
   const int b = find_sequence(p.cu, p.batch, t);
-  const int s0 = p.cu[b];
+  const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
   const int pos = t - s0, qb = pos / BS;
   const int slot0 = seq_first_slot(p.cu, b);
 
@@ -52,62 +52,86 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
   const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
   const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
 
-  for (int e = 0; e < p.topk; e++) {
-    const int blk = ip[(long long)e * p.isk];
-    if (blk < 0 || blk > qb) continue;
-    const int key0 = blk * BS;
-    f32x4 s[NSUB];
+  const int last_slot = (len - 1) >> 5;  // last slot of this sequence that exists in the copies
+  // the row of block ids is read once, 64 entries at a time (lane e holds entry e); the valid
+  // ones are then visited through a wave-uniform bit mask, so no load sits between two blocks
+  for (int e0 = 0; e0 < p.topk; e0 += 64) {
+  const int my_e = e0 + lane;
+  const int my_blk = my_e < p.topk ? ip[(long long)my_e * p.isk] : -1;
+  unsigned long long todo = __ballot(my_blk >= 0 && my_blk <= qb);
+  while (todo) {
+    const int e = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    const int blk = __builtin_amdgcn_readlane(my_blk, e);
+    // a block is walked in slices of up to 64 keys: all 2*NS*NK + NC*NDT fragment loads of a slice
+    // are issued back to back (no branches in between) so that ~32 KiB per wave are in flight
 #pragma unroll
-    for (int nt = 0; nt < NSUB; nt++) {
-      // fragment (slot, sub, kk) of the row-fragment copy: 512 elements each
-      const T* kp = kbase + (long long)(((key0 >> 4) + nt) * NK) * 512;
-      f32x4 c = {0.f, 0.f, 0.f, 0.f};
-      if (key0 + 16 * nt <= pos) {  // wave-uniform: sub-tiles wholly in the future are never loaded
+    for (int sl = 0; sl < (BS + 63) / 64; sl++) {
+      const int key0 = blk * BS + 64 * sl;
+      if (key0 > pos) break;
+      constexpr int NS = BS >= 64 ? 4 : BS / 16, NC = NS / 2;
+      v8 kfr[NS][NK], vfr[NC][NDT];
 #pragma unroll
-        for (int kk = 0; kk < NK; kk++) c = E::mfma16(ld16<v8>(kp + kk * 512), qf[kk], c);
+      for (int nt = 0; nt < NS; nt++) {
+        // sub-tiles wholly in the future are masked below; clamp them onto storage that exists
+        const int st = min((key0 >> 4) + nt, 2 * last_slot + 1);
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512);
       }
-      s[nt] = c;
+#pragma unroll
+      for (int c = 0; c < NC; c++) {
+        const int slot = min((key0 >> 5) + c, last_slot);
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) vfr[c][dt] = ld16<v8>(vbase + (long long)slot * D * 32 + dt * 512);
+      }
+      f32x4 s[NS];
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++) {
+        f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) c = E::mfma16(kfr[nt][kk], qf[kk], c);
+        s[nt] = c;
+      }
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int key = key0 + 16 * nt + 4 * lg + r;
+          const float x = key <= pos ? s[nt][r] * p.qk_scale : -INFINITY;
+          s[nt][r] = x;
+          mloc = fmaxf(mloc, x);
+        }
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      const float m_new = fmaxf(m, mloc);  // finite: key0 <= pos is always visible
+      const float alpha = fast_exp2(m - m_new);
+      m = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float x = fast_exp2(s[nt][r] - m_new);
+          s[nt][r] = x;
+          psum += x;
+        }
+      lsum = lsum * alpha + psum;
+#pragma unroll
+      for (int i = 0; i < NDT; i++) acc[i] *= alpha;
+#pragma unroll
+      for (int c = 0; c < NC; c++) {
+        v8 pf;  // probabilities of masked keys are exactly 0, the clamped V data they meet is finite
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          pf[r] = (T)s[2 * c][r];
+          pf[4 + r] = (T)s[2 * c + 1][r];
+        }
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) acc[dt] = E::mfma16(vfr[c][dt], pf, acc[dt]);
+      }
     }
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int nt = 0; nt < NSUB; nt++)
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        int key = key0 + 16 * nt + 4 * lg + r;
-        float x = key <= pos ? s[nt][r] * p.qk_scale : -INFINITY;
-        s[nt][r] = x;
-        mloc = fmaxf(mloc, x);
-      }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float m_new = fmaxf(m, mloc);  // finite: key0 <= pos is always visible
-    const float alpha = fast_exp2(m - m_new);
-    m = m_new;
-    float psum = 0.f;
-#pragma unroll
-    for (int nt = 0; nt < NSUB; nt++)
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        float x = fast_exp2(s[nt][r] - m_new);
-        s[nt][r] = x;
-        psum += x;
-      }
-    lsum = lsum * alpha + psum;
-#pragma unroll
-    for (int i = 0; i < NDT; i++) acc[i] *= alpha;
-#pragma unroll
-    for (int c = 0; c < NCH; c++) {
-      if (key0 + 32 * c > pos) break;  // wholly masked chunk: its slot of the transposed copy may not exist
-      v8 pf;
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        pf[r] = (T)s[2 * c][r];
-        pf[4 + r] = (T)s[2 * c + 1][r];
-      }
-      const T* vp = vbase + (long long)((key0 >> 5) + c) * D * 32;
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++) acc[dt] = E::mfma16(ld16<v8>(vp + dt * 512), pf, acc[dt]);
-    }
+  }
   }
   lsum += __shfl_xor(lsum, 16);
   lsum += __shfl_xor(lsum, 32);
