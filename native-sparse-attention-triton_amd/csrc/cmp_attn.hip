@@ -591,7 +591,7 @@ static int run_cmp(CmpArgs& a) {
     d.partial = (float*)(a.ws + L.partial);
     d.total_len = (int)a.Tq; d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;
     d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st;
-    d.qsn = a.p.qsn; d.qsh = a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = a.p.dsn; d.dsh = a.p.dsh;
+    d.qsn = (int)a.p.qsn; d.qsh = (int)a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = (int)a.p.dsn; d.dsh = (int)a.p.dsh;
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
     dkdv_kernel<T, D, 64, true><<<(unsigned)L.max_items, 256, 0, a.stream>>>(d);
     dkdv_reduce_kernel<T, D, 64><<<(unsigned)n_seg, 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
@@ -619,7 +619,7 @@ static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, c
                       int dtype, void* stream) {
   if (!q || !k || !cu_q || !cu_k || !strides || Tq <= 0 || Tk < 0 || B <= 0 || Hkv <= 0 || Hq % Hkv != 0 || ks <= 0 || st <= 0) return NSA_ERR_BAD_ARG;
   if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
-  for (int i = 0; i < 6; i++) if (strides[i] % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  for (int i = 0; i < 6; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 != 0) return NSA_ERR_UNSUPPORTED;
   CmpParams& p = a.p;
   p.q = q; p.k = k; p.v = v; p.cu_q = cu_q; p.cu_k = cu_k; p.total_q = (int)Tq; p.batch = (int)B; p.Hkv = (int)Hkv;
@@ -684,7 +684,7 @@ extern "C" int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, con
   int rc = cmp_common(a, q, k, v, cu_seqlens_q, cu_seqlens_k, total_q, total_k, batch, num_q_heads, num_kv_heads, kernel_size, kernel_stride, strides, sm_scale, dtype, stream);
   if (rc != NSA_OK) return rc;
   if (!v || !o || !dout || !lse || !dq || !dk || !dv || !workspace) return NSA_ERR_BAD_ARG;
-  for (int i = 6; i < 10; i++) if (strides[i] % 8 != 0) return NSA_ERR_UNSUPPORTED;
+  for (int i = 6; i < 10; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
   for (int i = 10; i < 16; i++) if (strides[i] % 4 != 0) return NSA_ERR_UNSUPPORTED;
   if (((uintptr_t)o | (uintptr_t)dout) % 16 != 0 || ((uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) % 8 != 0 || (uintptr_t)workspace % 256 != 0) return NSA_ERR_UNSUPPORTED;
   if (workspace_bytes < nsa_cmp_attn_bwd_workspace_bytes(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;

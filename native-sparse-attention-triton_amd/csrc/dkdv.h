@@ -15,6 +15,13 @@
 
 static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
 
+// LDS row that holds head hd of a staged 16-head row group.  The transposed reads of one
+// half-wave address the rows of heads {4*lg + j : lg in {0,1}, j < 4} (the other half-wave those of
+// lg in {2,3}); with the 272-byte row pitch these must be even (odd) rows to fall on 32 different
+// 8-byte bank pairs.  The plain 16-byte fragment reads touch all 16 rows and stay conflict-free
+// under any permutation.
+__device__ __forceinline__ int lds_row_of_head(int hd) { return ((((hd >> 2) & 1) * 4 + (hd & 3)) << 1) | (hd >> 3); }
+
 // chunk_off = exclusive scan of ceil((seg_end - seg_begin)/CHUNK_TOKENS) over segments (single workgroup).
 static __global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* __restrict__ seg_begin, const int32_t* __restrict__ seg_end, int n_seg,
                                                           int32_t* __restrict__ chunk_off) {
@@ -45,7 +52,8 @@ struct DkdvParams {
   const int32_t* cu; const int32_t* cu_k; const int32_t* cu_blk; const int32_t* seg_begin; const int32_t* seg_end; const int32_t* chunk_off; const int32_t* queries;
   float* partial;
   int total_len, batch, Hkv, G, GT, max_blocks, n_seg, ks, st;
-  long long qsn, qsh, ksn, ksh, vsn, vsh, dsn, dsh;
+  long long ksn, ksh, vsn, vsh;
+  int qsn, qsh, dsn, dsh;  // element strides of q / dO (checked on the host to fit 31 bits)
   float qk_scale, sm_scale;
 };
 
@@ -60,7 +68,7 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
   constexpr int LD = D + 8;                   // padded LDS row (elements)
   __shared__ __attribute__((aligned(16))) T q_s[2][2][16][LD];
   __shared__ __attribute__((aligned(16))) T do_s[2][2][16][LD];
-  __shared__ float lse_s[2][32], delta_s[2][32];
+  __shared__ __attribute__((aligned(16))) float lse_s[2][32], delta_s[2][32];
   __shared__ int pos_s[2][2];
 
   const int total_items = p.chunk_off[p.n_seg];
@@ -162,8 +170,8 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
         uint4 a = sg.qd[u], b2 = sg.dd[u];
         a.x &= m; a.y &= m; a.z &= m; a.w &= m;
         b2.x &= m; b2.y &= m; b2.z &= m; b2.w &= m;
-        *reinterpret_cast<uint4*>(&q_s[buf][rg][hd][8 * c]) = a;
-        *reinterpret_cast<uint4*>(&do_s[buf][rg][hd][8 * c]) = b2;
+        *reinterpret_cast<uint4*>(&q_s[buf][rg][lds_row_of_head(hd)][8 * c]) = a;
+        *reinterpret_cast<uint4*>(&do_s[buf][rg][lds_row_of_head(hd)][8 * c]) = b2;
       }
     }
     if (tid < 32) {
@@ -187,18 +195,20 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < NK; kk++) {
-          v8 qa = ld16<v8>(&q_s[buf][tk][li][32 * kk + 8 * lg]);
-          v8 da = ld16<v8>(&do_s[buf][tk][li][32 * kk + 8 * lg]);
+          v8 qa = ld16<v8>(&q_s[buf][tk][lds_row_of_head(li)][32 * kk + 8 * lg]);
+          v8 da = ld16<v8>(&do_s[buf][tk][lds_row_of_head(li)][32 * kk + 8 * lg]);
           s = E::mfma16(qa, kf[j][kk], s);
           dp = E::mfma16(da, vf[j][kk], dp);
         }
         const int pos = pos_s[buf][tk];
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[buf][tk * 16 + 4 * lg]);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_s[buf][tk * 16 + 4 * lg]);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float l2 = lse_s[buf][tk * 16 + 4 * lg + r];
-          const float dl = delta_s[buf][tk * 16 + 4 * lg + r];
+          const float l2 = l4[r];
+          const float dl = d4[r];
           const bool vis = RANGE ? (key < len && key * p.st + p.ks - 1 <= pos) : key <= pos;
-          const float pr = vis ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
+          const float pr = fast_exp2(vis ? s[r] * p.qk_scale - l2 : -INFINITY);  // select, not a branch
           pf[j][tk * 4 + r] = (T)pr;
           dsf[j][tk * 4 + r] = (T)(pr * (dp[r] - dl) * p.sm_scale);
         }
@@ -214,8 +224,8 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
       s16x8 qt, dot;
 #pragma unroll
       for (int tk = 0; tk < 2; tk++) {
-        const T* qa = &q_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
-        const T* da = &do_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+        const T* qa = &q_s[buf][tk][lds_row_of_head(4 * lg + (li >> 2))][16 * dt + 4 * (li & 3)];
+        const T* da = &do_s[buf][tk][lds_row_of_head(4 * lg + (li >> 2))][16 * dt + 4 * (li & 3)];
         s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(qa));
         s16x4 c = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(da));
 #pragma unroll

@@ -291,7 +291,7 @@ static int run_bwd(const BwdArgs& a) {
     p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.vals_out);
     p.partial = (float*)(ws + L.partial);
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
-    p.qsn = a.qsn; p.qsh = a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = a.dsn; p.dsh = a.dsh;
+    p.qsn = (int)a.qsn; p.qsh = (int)a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = (int)a.dsn; p.dsh = (int)a.dsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1;
     constexpr int NT = (BS / 16 < 4 ? BS / 16 : 4) * 64;
     dkdv_kernel<T, D, BS, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
@@ -356,7 +356,7 @@ extern "C" int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, co
   if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
   if ((out_segment_offsets == nullptr) != (out_queries == nullptr)) return NSA_ERR_BAD_ARG;
   if (num_kv_heads * total_len * topk >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
-  for (int i = 0; i < 10; i++) if (strides[i] % 8 != 0) return NSA_ERR_UNSUPPORTED;       // 16-byte loads
+  for (int i = 0; i < 10; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;  // 16-byte loads, 31-bit strides
   for (int i = 13; i < 19; i++) if (strides[i] % 4 != 0) return NSA_ERR_UNSUPPORTED;      // 8-byte stores
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)dout) % 16 != 0) return NSA_ERR_UNSUPPORTED;
   if (((uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) % 8 != 0 || (uintptr_t)workspace % 256 != 0) return NSA_ERR_UNSUPPORTED;
