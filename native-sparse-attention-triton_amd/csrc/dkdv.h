@@ -57,7 +57,8 @@ struct DkdvParams {
   float qk_scale, sm_scale;
 };
 
-template <typename T, int D, int BS, bool RANGE>
+// GT1: the GQA group has at most 16 query heads (one head tile), which removes every run-time division
+template <typename T, int D, int BS, bool RANGE, bool GT1>
 __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_kernel(DkdvParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
@@ -88,7 +89,8 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
   const int key0 = (gb - p.cu_blk[b]) * BS;
   const int first = p.seg_begin[seg] + (item - p.chunk_off[seg]) * CHUNK_TOKENS;
   const int n_tok = min(CHUNK_TOKENS, p.seg_end[seg] - first);
-  const int n_rg = n_tok * p.GT;              // row groups (token, head tile) in this chunk
+  const int GT = GT1 ? 1 : p.GT;
+  const int n_rg = n_tok * GT;                // row groups (token, head tile) in this chunk
   const int n_step = (n_rg + 1) / 2;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -139,8 +141,8 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
       const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = pc / (D / 8) / 16;
       const int r = step * 2 + rg;
       const int rc = min(r, n_rg - 1);
-      const int t = tok_s[rc / p.GT];
-      const int hq = (rc % p.GT) * 16 + hd;
+      const int t = tok_s[GT1 ? rc : rc / GT];
+      const int hq = (GT1 ? 0 : (rc % GT) * 16) + hd;
       const int hc = min(hq, p.G - 1);
       sg.qd[u] = *reinterpret_cast<const uint4*>(qbase + (long long)t * p.qsn + (long long)hc * p.qsh + 8 * c);
       sg.dd[u] = *reinterpret_cast<const uint4*>(dbase + (long long)t * p.dsn + (long long)hc * p.dsh + 8 * c);
@@ -150,8 +152,8 @@ __global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_k
       const int rg = (tid >> 4) & 1, hd = tid & 15;
       const int r = step * 2 + rg;
       const int rc = min(r, n_rg - 1);
-      const int t = tok_s[rc / p.GT];
-      const int hq = (rc % p.GT) * 16 + hd;
+      const int t = tok_s[GT1 ? rc : rc / GT];
+      const int hq = (GT1 ? 0 : (rc % GT) * 16) + hd;
       const int hc = min(hq, p.G - 1);
       sg.lse = lbase[(long long)hc * p.total_len + t];
       sg.delta = ebase[(long long)hc * p.total_len + t];
