@@ -66,6 +66,168 @@ def cpu_baseline():
     }
 
 
+def _time_ms(fn, iters, warm=2):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    return _events_ms(fn, iters)
+
+
+def bench_pipeline(args, dev):
+    """BASELINE config 1: linear_compress -> compressed_attention (+selection) -> topk_sparse_attention, forward, bf16."""
+    from native_sparse_attention.ops import compressed_attention, linear_compress, topk_sparse_attention
+    from native_sparse_attention.ops.compressed_attention import _compressed_attention_fwd, _select_blocks
+    from native_sparse_attention.testing import cu_from_lens
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    cu = cu_from_lens([1024, 7168, 8192], dev)
+    T, ks, st, bs, topk = 16384, 32, 16, 64, 16
+    q = torch.randn(T, HQ, D, generator=g, device=dev).bfloat16()
+    k = torch.randn(T, HKV, D, generator=g, device=dev).bfloat16()
+    v = torch.randn(T, HKV, D, generator=g, device=dev).bfloat16()
+    wk = (torch.randn(HKV, ks * D, D, generator=g, device=dev) / (ks * D) ** 0.5).bfloat16()
+    wv = (torch.randn(HKV, ks * D, D, generator=g, device=dev) / (ks * D) ** 0.5).bfloat16()
+    pe = (0.02 * torch.randn(HKV, ks, D, generator=g, device=dev)).bfloat16()
+    it = args.steps
+    with torch.no_grad():
+        ck, cuk = linear_compress(k, wk, cu, ks, st, pe)
+        cv, _ = linear_compress(v, wv, cu, ks, st)
+        o_c, idx = compressed_attention(q, ck, cv, ks, st, bs, topk, cu, cuk, 8192, 511)
+        o_c2, lse = _compressed_attention_fwd(q, ck, cv, ks, st, cu, cuk, 8192, 511, D ** -0.5)
+        t_lin = _time_ms(lambda: (linear_compress(k, wk, cu, ks, st, pe), linear_compress(v, wv, cu, ks, st)), it)
+        t_cmp = _time_ms(lambda: _compressed_attention_fwd(q, ck, cv, ks, st, cu, cuk, 8192, 511, D ** -0.5), it)
+        t_sel = _time_ms(lambda: _select_blocks(q, ck, lse, ks, st, bs, topk, cu, cuk, 8192, 1, 2, D ** -0.5), it)
+        t_top = _time_ms(lambda: topk_sparse_attention(q, k, v, idx, bs, cu), it)
+
+        def whole():
+            a, c = linear_compress(k, wk, cu, ks, st, pe)
+            b, _ = linear_compress(v, wv, cu, ks, st)
+            _, i2 = compressed_attention(q, a, b, ks, st, bs, topk, cu, c, 8192, 511)
+            return topk_sparse_attention(q, k, v, i2, bs, cu)
+        t_all = _time_ms(whole, it)
+    lens = [1024, 7168, 8192]
+    pairs = sum(sum((i - ks + 1) // st + 1 for i in range(ks - 1, L)) for L in lens)
+    f_lin = 2 * 2.0 * int(cuk[-1]) * ks * D * D * HKV
+    f_cmp = 4.0 * D * HQ * pairs
+    f_top = 4.0 * D * bs * (HQ // HKV) * int((idx >= 0).sum())
+    return {
+        "metric": "NSA op pipeline forward ms (linear_compress x2 + compressed_attention w/ selection + topk_sparse_attention)",
+        "value": t_all, "unit": "ms", "n_gpus": 1, "steps": it, "warmup": 2, "ms_per_step": t_all, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cu_seqlens=[0,1024,8192,16384], 64q/4kv heads, d=128, kernel 32 stride 16, block 64, top-16",
+                   "ms": {"linear_compress_kv": t_lin, "compressed_attention_fwd": t_cmp, "block_selection": t_sel, "topk_sparse_attention_fwd": t_top},
+                   "tflops": {"linear_compress_kv": f_lin / t_lin / 1e9, "compressed_attention_fwd": f_cmp / t_cmp / 1e9,
+                              "topk_sparse_attention_fwd": f_top / t_top / 1e9}},
+    }
+
+
+def bench_compressed(args, dev):
+    """BASELINE config 3: weightedpool compression + compressed_attention forward+backward, N=65536, 32q/2kv."""
+    from native_sparse_attention.ops import compressed_attention, weightedpool_compress
+    from native_sparse_attention.ops.compressed_attention import _compressed_attention_bwd, _compressed_attention_fwd, _select_blocks
+    from native_sparse_attention.testing import cu_from_lens
+
+    N, Hq, Hkv, ks, st, bs, topk = 65536, 32, 2, 32, 16, 64, 16
+    g = torch.Generator(device=dev).manual_seed(0)
+    cu = cu_from_lens([N], dev)
+    q = torch.randn(N, Hq, D, generator=g, device=dev).bfloat16().requires_grad_()
+    k = torch.randn(N, Hkv, D, generator=g, device=dev).bfloat16().requires_grad_()
+    v = torch.randn(N, Hkv, D, generator=g, device=dev).bfloat16().requires_grad_()
+    wk = torch.softmax(torch.randn(Hkv, ks, generator=g, device=dev), -1).bfloat16().requires_grad_()
+    wv = torch.softmax(torch.randn(Hkv, ks, generator=g, device=dev), -1).bfloat16().requires_grad_()
+    do = torch.randn(N, Hq, D, generator=g, device=dev).bfloat16()
+    it = max(2, min(args.steps, 5))
+
+    def step():
+        ck, cuk = weightedpool_compress(k, wk, cu, ks, st)
+        cv, _ = weightedpool_compress(v, wv, cu, ks, st)
+        o, idx = compressed_attention(q, ck, cv, ks, st, bs, topk, cu, cuk, N, 4095)
+        o.backward(do)
+        return idx
+    t_all = _time_ms(step, it, warm=1)
+    with torch.no_grad():
+        ck, cuk = weightedpool_compress(k, wk, cu, ks, st)
+        cv, _ = weightedpool_compress(v, wv, cu, ks, st)
+        o, lse = _compressed_attention_fwd(q, ck, cv, ks, st, cu, cuk, N, 4095, D ** -0.5)
+        t_pool = _time_ms(lambda: weightedpool_compress(k, wk, cu, ks, st), it)
+        t_fwd = _time_ms(lambda: _compressed_attention_fwd(q, ck, cv, ks, st, cu, cuk, N, 4095, D ** -0.5), it)
+        t_sel = _time_ms(lambda: _select_blocks(q, ck, lse, ks, st, bs, topk, cu, cuk, N, 1, 2, D ** -0.5), it)
+        t_bwd = _time_ms(lambda: _compressed_attention_bwd(o, do, lse, q, ck, cv, ks, st, cu, cuk, N, 4095, D ** -0.5), it)
+    pairs = sum((i - ks + 1) // st + 1 for i in range(ks - 1, N))
+    f_fwd = 4.0 * D * Hq * pairs
+    pool_bytes = (N * Hkv * D + 4095 * Hkv * D) * 2
+    return {
+        "metric": "weightedpool + compressed_attention fwd+bwd ms (N=65536)", "value": t_all, "unit": "ms", "n_gpus": 1, "steps": it,
+        "warmup": 1, "ms_per_step": t_all, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "single sequence N=65536, 32q/2kv heads, d=128, kernel 32 stride 16, block 64, top-16",
+                   "ms": {"weightedpool_fwd_one_tensor": t_pool, "compressed_attention_fwd": t_fwd, "block_selection": t_sel,
+                          "compressed_attention_bwd": t_bwd},
+                   "tflops": {"compressed_attention_fwd": f_fwd / t_fwd / 1e9, "compressed_attention_bwd": 2.5 * f_fwd / t_bwd / 1e9},
+                   "gbps": {"weightedpool_fwd": pool_bytes / t_pool / 1e6}},
+    }
+
+
+def bench_decode(args, dev):
+    """BASELINE config 4: one NSA decode step over the cache slabs (three branches + sigmoid gates)."""
+    from native_sparse_attention.infer import nsa_infer
+    from native_sparse_attention.module import NSACache
+    from native_sparse_attention.ops import weightedpool_compress
+    from native_sparse_attention.testing import cu_from_lens
+
+    Hq, Hkv, ks, st, bs, topk, W = 32, 2, 32, 16, 64, 8, 512
+    lens = [2048, 4096, 6144, 8192]
+    B = len(lens)
+    g = torch.Generator(device=dev).manual_seed(0)
+    cu = cu_from_lens(lens, dev)
+    T = int(cu[-1])
+    q = torch.randn(T, Hq, D, generator=g, device=dev).bfloat16()
+    k = torch.randn(T, Hkv, D, generator=g, device=dev).bfloat16()
+    v = torch.randn(T, Hkv, D, generator=g, device=dev).bfloat16()
+    gate = torch.sigmoid(torch.randn(T, Hq, 3, generator=g, device=dev)).bfloat16()
+    wk = torch.softmax(torch.randn(Hkv, ks, generator=g, device=dev), -1).bfloat16()
+    wv = torch.softmax(torch.randn(Hkv, ks, generator=g, device=dev), -1).bfloat16()
+    rope = lambda x, c, s, stride=1: x
+    steps = max(4, args.steps)
+    cache = NSACache(B, max(lens) + steps + 8, Hkv, D, ks, st, W, torch.bfloat16, dev)
+    fargs = (rope, cache, (wk, wv), (weightedpool_compress, weightedpool_compress), None, ks, st, bs, topk, 1, 2, W)
+    with torch.no_grad():
+        nsa_infer(cu, 0, q, k, v, gate, *fargs)
+        qd = torch.randn(B, Hq, D, generator=g, device=dev).bfloat16()
+        kd = torch.randn(B, Hkv, D, generator=g, device=dev).bfloat16()
+        vd = torch.randn(B, Hkv, D, generator=g, device=dev).bfloat16()
+        gd = torch.sigmoid(torch.randn(B, Hq, 3, generator=g, device=dev)).bfloat16()
+        nsa_infer(cu, 1, qd, kd, vd, gd, *fargs)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for s in range(2, steps + 2):
+            nsa_infer(cu, s, qd, kd, vd, gd, *fargs)
+        torch.cuda.synchronize()
+        us = (time.perf_counter() - t0) * 1e6 / steps
+        # the three attention kernels alone, on the final cache state
+        from native_sparse_attention.ops import compressed_attention_decode, flash_attention_decode, topk_sparse_attention_decode
+        seqlens = cache.sparse_kv_len[:B].clone()
+        rows = int(cache.compress_kv_len[:B].max())
+        o1, idx = compressed_attention_decode(qd, cache.compress_kv_cache[0, :B, :rows], cache.compress_kv_cache[1, :B, :rows],
+                                              seqlens, cache.compress_kv_len[:B], ks, st, bs, topk)
+        t_c = _time_ms(lambda: compressed_attention_decode(qd, cache.compress_kv_cache[0, :B, :rows], cache.compress_kv_cache[1, :B, :rows],
+                                                           seqlens, cache.compress_kv_len[:B], ks, st, bs, topk), 20)
+        t_s = _time_ms(lambda: topk_sparse_attention_decode(qd, cache.sparse_kv_cache[0, :B], cache.sparse_kv_cache[1, :B], idx, bs, seqlens), 20)
+        wl = torch.clamp(cache.sliding_kv_len[:B], max=W)
+        t_w = _time_ms(lambda: flash_attention_decode(qd, cache.sliding_kv_cache[0, :B], cache.sliding_kv_cache[1, :B], wl), 20)
+    key_rows = int(cache.compress_kv_len[:B].sum()) + 64 * int((idx >= 0).sum()) // Hkv + B * W
+    alg_bytes = 2 * Hkv * D * 2 * key_rows
+    return {
+        "metric": "NSA decode step latency (us), B=4, cached lens 2K..8K", "value": us, "unit": "us", "n_gpus": 1, "steps": steps,
+        "warmup": 2, "ms_per_step": us / 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "32q/2kv heads, d=128, weightedpool kernel 32 stride 16, block 64, top-8, window 512, sigmoid gates",
+                   "us": {"full_step_incl_cache_update_and_compress": us, "compressed_decode_with_selection": t_c * 1e3,
+                          "topk_decode": t_s * 1e3, "window_decode": t_w * 1e3},
+                   "algorithmic_kv_bytes": alg_bytes, "gbps_three_kernels": alg_bytes / ((t_c + t_s + t_w) * 1e-3) / 1e9},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,6 +236,8 @@ def main():
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--topk", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode"],
+                    help="topk = the headline metric (default); the others time BASELINE configs 1, 3 and 4")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the operator path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -85,6 +249,10 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload != "topk":
+        fn = {"pipeline": bench_pipeline, "compressed": bench_compressed, "decode": bench_decode}[args.workload]
+        print(json.dumps(fn(args, dev)))
+        return
     N, topk = args.seqlen, args.topk
     G = HQ // HKV
     g = torch.Generator(device=dev).manual_seed(0)
