@@ -593,8 +593,8 @@ static int run_cmp(CmpArgs& a) {
     d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st;
     d.qsn = (int)a.p.qsn; d.qsh = (int)a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = (int)a.p.dsn; d.dsh = (int)a.p.dsh;
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
-    if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items, 256, 0, a.stream>>>(d);
-    else dkdv_kernel<T, D, 64, true, false><<<(unsigned)L.max_items, 256, 0, a.stream>>>(d);
+    if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
+    else dkdv_kernel<T, D, 64, true, false><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
     dkdv_reduce_kernel<T, D, 64><<<(unsigned)n_seg, 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
                                                                        (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
     a.p.delta = delta;

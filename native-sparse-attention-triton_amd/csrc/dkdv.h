@@ -15,6 +15,11 @@
 
 static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
 
+// Waves per dK/dV workgroup; each wave owns bs / (16 * waves) key tiles.  Every wave reads all
+// staged query rows from LDS, so fewer waves would mean fewer LDS reads per token, but two waves
+// of 32 keys need > 256 registers each (one wave per SIMD) and measured 17% slower than four.
+constexpr int dkdv_waves(int bs) { return bs >= 64 ? 4 : bs / 16; }
+
 // LDS row that holds head hd of a staged 16-head row group.  The transposed reads of one
 // half-wave address the rows of heads {4*lg + j : lg in {0,1}, j < 4} (the other half-wave those of
 // lg in {2,3}); with the 272-byte row pitch these must be even (odd) rows to fall on 32 different
@@ -59,11 +64,11 @@ struct DkdvParams {
 
 // GT1: the GQA group has at most 16 query heads (one head tile), which removes every run-time division
 template <typename T, int D, int BS, bool RANGE, bool GT1>
-__global__ __launch_bounds__(BS >= 64 ? 256 : 128, BS <= 64 ? 2 : 1) void dkdv_kernel(DkdvParams p) {
+__global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_kernel(DkdvParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16;
-  constexpr int NW = NSUB < 4 ? NSUB : 4;     // waves per workgroup
+  constexpr int NW = dkdv_waves(BS);          // waves per workgroup
   constexpr int KT = NSUB / NW;               // 16-key tiles per wave
   constexpr int NT = NW * 64;
   constexpr int LD = D + 8;                   // padded LDS row (elements)
