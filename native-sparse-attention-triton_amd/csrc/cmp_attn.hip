@@ -595,7 +595,7 @@ static int run_cmp(CmpArgs& a) {
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
     if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
     else dkdv_kernel<T, D, 64, true, false><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
-    dkdv_reduce_kernel<T, D, 64><<<(unsigned)n_seg, 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
+    dkdv_reduce_kernel<T, D, 64><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
                                                                        (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
     a.p.delta = delta;
     cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);

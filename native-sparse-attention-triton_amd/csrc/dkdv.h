@@ -286,7 +286,8 @@ __global__ __launch_bounds__(256) void dkdv_reduce_kernel(const float* __restric
   const int s0 = cu[b], len = cu[b + 1] - s0;
   const int key0 = (gb - cu_blk[b]) * BS;
   const int c0 = chunk_off[seg], c1 = chunk_off[seg + 1];
-  for (int i = threadIdx.x; i < 2 * BS * (D / 4); i += 256) {
+  // blockIdx.y splits the 2*BS*D/4 output pieces of a segment so that short segments still fill the chip
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < 2 * BS * (D / 4); i += 256 * gridDim.y) {
     const int which = i / (BS * (D / 4)), key = (i / (D / 4)) % BS, d4 = i % (D / 4);
     if (key0 + key >= len) continue;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};

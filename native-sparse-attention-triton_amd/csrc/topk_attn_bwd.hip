@@ -296,7 +296,7 @@ static int run_bwd(const BwdArgs& a) {
     constexpr int NT = 64 * dkdv_waves(BS);
     if (GT == 1) dkdv_kernel<T, D, BS, false, true><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
     else dkdv_kernel<T, D, BS, false, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
-    dkdv_reduce_kernel<T, D, BS><<<(unsigned)n_seg, 256, 0, a.stream>>>(
+    dkdv_reduce_kernel<T, D, BS><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(
         p.partial, p.chunk_off, a.cu, p.cu_blk, (int)a.B, (int)L.max_blocks, (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
   }
   if (a.phases & NSA_BWD_PHASE_DQ) {
