@@ -26,6 +26,9 @@ PEAK_BF16_TFLOPS = 2500.0        # MI355X dense bf16 MFMA
 HQ, HKV, D, BS = 64, 4, 128, 64
 # reference-published Triton timings for this exact workload (its README.md:219,229): H100 fwd + bwd, ms
 H100_FWD_BWD_MS = 12.417 + 15.154
+# memory-side traffic per launch at the default workload (N=32768, top16), bytes: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, scaled by what the same counters read for a plain 1 GiB copy (x2.0 and x1.0); see profiles/
+MEASURED_TRAFFIC = {"fwd_attend": 20.0 * 2**30, "bwd_dq": 18.2 * 2**30, "bwd_dkdv": 18.1 * 2**30}
 
 
 def _events_ms(fn, iters):
@@ -236,6 +239,8 @@ def main():
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--topk", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 1 GiB device copies (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode"],
                     help="topk = the headline metric (default); the others time BASELINE configs 1, 3 and 4")
     args = ap.parse_args()
@@ -311,12 +316,20 @@ def main():
             "baseline": "H100 Triton fwd+bwd ms published in the reference README (12.417 + 15.154)",
             "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "frac_of_bf16_peak": f_total / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
             "kernel_ms": {n: kern[n][0] for n in kern},
+            "kernel_tflops": {n: kern[n][1] / kern[n][0] / 1e9 for n in kern if kern[n][1] > 0},
         },
         "roofline": {
             "bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+            "frac": achieved / PEAK_BF16_TFLOPS,
+            "traffic": MEASURED_TRAFFIC.get(dom) if (N, topk) == (32768, 16) else None,
         },
     }
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # 1 GiB read + 1 GiB written per launch
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
