@@ -160,15 +160,16 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   }
   const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
   const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
-  Stager<T, D, 2> stg;
+  // two register stages with fixed roles (the loop is unrolled by two): chunk ch+2 is requested while
+  // chunk ch is being consumed, so a full chunk of compute hides each load
+  Stager<T, D, 2> stg0, stg1;
   if (n_chunks > ch0) {
-    stg.fetch(kb, p.ksn, vb, p.vsn, ch0, ti.lk, tid);
-    stg.stash(k_s[0], v_s[0], tid);
+    stg0.fetch(kb, p.ksn, vb, p.vsn, ch0, ti.lk, tid);
+    stg0.stash(k_s[0], v_s[0], tid);
+    stg1.fetch(kb, p.ksn, vb, p.vsn, min(ch0 + 1, n_chunks - 1), ti.lk, tid);
   }
   __syncthreads();
-  for (int ch = ch0; ch < n_chunks; ch++) {
-    const int buf = (ch - ch0) & 1;
-    if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, vb, p.vsn, ch + 1, ti.lk, tid);
+  auto compute = [&](const int ch, const int buf) {
     if (32 * ch < wave_hi && 32 * ch + 32 > wave_lo) {
       f32x4 s[4][2];
 #pragma unroll
@@ -213,8 +214,11 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
             pf[j][4 * sub + r] = (T)x;
           }
         l[j] = l[j] * alpha + psum;
+        // the running maximum settles after the first chunks: skip the 4*NDT multiplies when no lane rescales
+        if (__ballot(alpha != 1.f)) {
 #pragma unroll
-        for (int i = 0; i < NDT; i++) acc[j][i] *= alpha;
+          for (int i = 0; i < NDT; i++) acc[j][i] *= alpha;
+        }
       }
 #pragma unroll
       for (int dt = 0; dt < NDT; dt++) {
@@ -223,8 +227,18 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
         for (int j = 0; j < 4; j++) acc[j][dt] = E::mfma16(vt, pf[j], acc[j][dt]);
       }
     }
-    if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], v_s[buf ^ 1], tid);
+  };
+  for (int ch = ch0; ch < n_chunks; ch += 2) {
+    stg0.fetch(kb, p.ksn, vb, p.vsn, min(ch + 2, n_chunks - 1), ti.lk, tid);
+    compute(ch, 0);
+    if (ch + 1 < n_chunks) stg1.stash(k_s[1], v_s[1], tid);
     __syncthreads();
+    if (ch + 1 < n_chunks) {
+      stg1.fetch(kb, p.ksn, vb, p.vsn, min(ch + 3, n_chunks - 1), ti.lk, tid);
+      compute(ch + 1, 1);
+      if (ch + 2 < n_chunks) stg0.stash(k_s[0], v_s[0], tid);
+      __syncthreads();
+    }
   }
 #pragma unroll
   for (int j = 0; j < 4; j++) {
@@ -295,15 +309,16 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
     for (int i = 0; i < NDT; i++) acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
   const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
   const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
-  Stager<T, D, 2> stg;
+  // two register stages with fixed roles (the loop is unrolled by two): chunk ch+2 is requested while
+  // chunk ch is being consumed, so a full chunk of compute hides each load
+  Stager<T, D, 2> stg0, stg1;
   if (n_chunks > 0) {
-    stg.fetch(kb, p.ksn, vb, p.vsn, 0, ti.lk, tid);
-    stg.stash(k_s[0], v_s[0], tid);
+    stg0.fetch(kb, p.ksn, vb, p.vsn, 0, ti.lk, tid);
+    stg0.stash(k_s[0], v_s[0], tid);
+    stg1.fetch(kb, p.ksn, vb, p.vsn, min(0 + 1, n_chunks - 1), ti.lk, tid);
   }
   __syncthreads();
-  for (int ch = 0; ch < n_chunks; ch++) {
-    const int buf = ch & 1;
-    if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, vb, p.vsn, ch + 1, ti.lk, tid);
+  auto compute = [&](const int ch, const int buf) {
     if (32 * ch < wave_lim) {
       v8 dsf[TPW];
 #pragma unroll
@@ -337,8 +352,18 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
         for (int j = 0; j < TPW; j++) acc[j][dt] = E::mfma16(kt, dsf[j], acc[j][dt]);
       }
     }
-    if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], v_s[buf ^ 1], tid);
+  };
+  for (int ch = 0; ch < n_chunks; ch += 2) {
+    stg0.fetch(kb, p.ksn, vb, p.vsn, min(ch + 2, n_chunks - 1), ti.lk, tid);
+    compute(ch, 0);
+    if (ch + 1 < n_chunks) stg1.stash(k_s[1], v_s[1], tid);
     __syncthreads();
+    if (ch + 1 < n_chunks) {
+      stg1.fetch(kb, p.ksn, vb, p.vsn, min(ch + 3, n_chunks - 1), ti.lk, tid);
+      compute(ch + 1, 1);
+      if (ch + 2 < n_chunks) stg0.stash(k_s[0], v_s[0], tid);
+      __syncthreads();
+    }
   }
 #pragma unroll
   for (int j = 0; j < TPW; j++) {
