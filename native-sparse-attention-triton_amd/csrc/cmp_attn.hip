@@ -13,6 +13,7 @@
 // reference): per token the probabilities are recomputed chunk by chunk from the final LSE,
 // summed over the group's heads, folded into block scores with the overlap weights, then the k
 // best blocks are extracted by repeated wave-wide arg-max and written in ascending order.
+#include <type_traits>
 #include "delta.h"
 #include "dkdv.h"
 
@@ -61,10 +62,10 @@ __device__ __forceinline__ void visible_range(int pos, int lq, int lk, int ks, i
 
 // stage rows [32*chunk, +32) of one or two [*, H, D] tensors into LDS tiles (zeros past lk).  The two
 // tensors are handled by separate unrolled loops (no run-time choice of the base pointer).
-template <typename T, int D, int NTENS>
+template <typename T, int D, int NTENS, int NT = 256>
 struct Stager {
   static constexpr int PIECES = 32 * (D / 8);  // per tensor
-  static constexpr int PPT = (PIECES + 255) / 256;
+  static constexpr int PPT = (PIECES + NT - 1) / NT;
   uint4 ra[PPT], rb[PPT];
   unsigned ok;
   // branch-free: always load (from a clamped row), mask when writing to LDS
@@ -72,7 +73,7 @@ struct Stager {
     ok = 0;
 #pragma unroll
     for (int u = 0; u < PPT; u++) {
-      const int pc = min(tid + u * 256, PIECES - 1);
+      const int pc = min(tid + u * NT, PIECES - 1);
       const int c = pc % (D / 8), r = pc / (D / 8);
       const int key = chunk * 32 + r;
       const int kc = min(key, lk - 1);
@@ -84,7 +85,7 @@ struct Stager {
   __device__ __forceinline__ void stash(T (*ta)[D + 8], T (*tb)[D + 8], int tid) {
 #pragma unroll
     for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * 256;
+      const int pc = tid + u * NT;
       if (pc < PIECES) {
         const int c = pc % (D / 8), r = pc / (D / 8);
         const unsigned m = 0u - ((ok >> u) & 1u);  // all ones when the row exists
@@ -101,6 +102,9 @@ struct Stager {
   }
 };
 
+// floor of the running score maxima (raw q.k units): finite, so differences of maxima never form inf - inf
+#define M_FLOOR (-1e30f)
+
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 // fragment of X^T for 16 columns starting at d0 over the 32 staged rows, in the k-order of the
@@ -116,12 +120,15 @@ __device__ __forceinline__ typename Elem<T>::v8 tr_frag(const T (*tile)[LD], int
 }
 
 // ------------------------------------------------------------------------------------------
+// tokens per wave of the forward kernel: two keeps a wave within 256 registers, so two waves share a
+// SIMD and one wave's softmax arithmetic overlaps the other's MFMAs
+constexpr int FWD_TPW = 2;
 template <typename T, int D>
-__global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
+__global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8;
+  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8, TPW = FWD_TPW, NT = 64 * (16 / TPW);
   __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
   __shared__ __attribute__((aligned(16))) T v_s[2][32][LD];
   TileInfo ti;
@@ -131,14 +138,16 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   const int hq = gt * 16 + li;
   const bool has_head = hq < p.G;
   const int hh = h * p.G + (has_head ? hq : 0);
-  v8 qf[4][NK];
-  int lo[4], hi[4];
-  int wave_lo = 1 << 30, wave_hi = 0;
+  v8 qf[TPW][NK];
+  int lo[TPW], hi[TPW];
+  int wave_lo = 1 << 30, wave_hi = 0, wave_lo_max = 0, wave_hi_min = 1 << 30;
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int pos = ti.i0 + 4 * wave + j;
+  for (int j = 0; j < TPW; j++) {
+    const int pos = ti.i0 + TPW * wave + j;
     visible_range(pos, ti.lq, ti.lk, p.ks, p.st, p.window, lo[j], hi[j]);
     wave_hi = max(wave_hi, hi[j]);
+    wave_hi_min = min(wave_hi_min, hi[j]);
+    wave_lo_max = max(wave_lo_max, lo[j]);
     if (hi[j] > 0) wave_lo = min(wave_lo, lo[j]);
     const bool live = has_head && pos < ti.lq;
     const T* qp = (const T*)p.q + (long long)(ti.s0q + (pos < ti.lq ? pos : 0)) * p.qsn + (long long)hh * p.qsh + 8 * lg;
@@ -150,11 +159,11 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   visible_range(ti.i0, ti.lq, ti.lk, p.ks, p.st, p.window, tile_lo, unused);
   const int ch0 = tile_lo / 32;                 // the first token of the tile reaches furthest back
   const int n_chunks = (tile_hi + 31) / 32;
-  f32x4 acc[4][NDT];
-  float m[4], l[4];
+  f32x4 acc[TPW][NDT];
+  float m[TPW], l[TPW];
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    m[j] = -INFINITY; l[j] = 0.f;
+  for (int j = 0; j < TPW; j++) {
+    m[j] = M_FLOOR; l[j] = 0.f;
 #pragma unroll
     for (int i = 0; i < NDT; i++) acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -162,7 +171,7 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
   // two register stages with fixed roles (the loop is unrolled by two): chunk ch+2 is requested while
   // chunk ch is being consumed, so a full chunk of compute hides each load
-  Stager<T, D, 2> stg0, stg1;
+  Stager<T, D, 2, NT> stg0, stg1;
   if (n_chunks > ch0) {
     stg0.fetch(kb, p.ksn, vb, p.vsn, ch0, ti.lk, tid);
     stg0.stash(k_s[0], v_s[0], tid);
@@ -171,60 +180,68 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
   __syncthreads();
   auto compute = [&](const int ch, const int buf) {
     if (32 * ch < wave_hi && 32 * ch + 32 > wave_lo) {
-      f32x4 s[4][2];
+      f32x4 s[TPW][2];
 #pragma unroll
       for (int sub = 0; sub < 2; sub++) {
         v8 kf[NK];
 #pragma unroll
         for (int kk = 0; kk < NK; kk++) kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < TPW; j++) {
           f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int kk = 0; kk < NK; kk++) c = E::mfma16(kf[kk], qf[j][kk], c);
           s[j][sub] = c;
         }
       }
-      v8 pf[4];
+      v8 pf[TPW];
+      // Running maxima are kept in raw score units with a finite floor, so a token that sees nothing
+      // yet needs no special case: exp2(-inf - finite) is 0 and the floor minus itself gives alpha 1.
+      auto softmax = [&](auto masked) {
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        float mloc = -INFINITY;
+        for (int j = 0; j < TPW; j++) {
+          float mloc = M_FLOOR;
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++)
+          for (int sub = 0; sub < 2; sub++)
 #pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const int c = 32 * ch + 16 * sub + 4 * lg + r;
-            const float x = (c >= lo[j] && c < hi[j]) ? s[j][sub][r] * p.qk_scale : -INFINITY;
-            s[j][sub][r] = x;
-            mloc = fmaxf(mloc, x);
+            for (int r = 0; r < 4; r++) {
+              if (decltype(masked)::value) {
+                const int c = 32 * ch + 16 * sub + 4 * lg + r;
+                if (!(c >= lo[j] && c < hi[j])) s[j][sub][r] = -INFINITY;
+              }
+              mloc = fmaxf(mloc, s[j][sub][r]);
+            }
+          mloc = column_max(mloc);
+          const float m_new = fmaxf(m[j], mloc);
+          const float alpha = fast_exp2((m[j] - m_new) * p.qk_scale);
+          const float mb = m_new * p.qk_scale;
+          m[j] = m_new;
+          float psum = 0.f;
+#pragma unroll
+          for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              const float x = fast_exp2(__builtin_fmaf(s[j][sub][r], p.qk_scale, -mb));
+              psum += x;
+              pf[j][4 * sub + r] = (T)x;
+            }
+          l[j] = l[j] * alpha + psum;
+          // the running maximum settles after the first chunks: skip the 4*NDT multiplies when no lane rescales
+          if (__ballot(alpha != 1.f)) {
+#pragma unroll
+            for (int i = 0; i < NDT; i++) acc[j][i] *= alpha;
           }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        const float m_new = fmaxf(m[j], mloc);
-        const bool dead = m_new == -INFINITY;  // nothing visible yet for this token
-        const float alpha = dead ? 1.f : fast_exp2(m[j] - m_new);
-        m[j] = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const float x = dead ? 0.f : fast_exp2(s[j][sub][r] - m_new);
-            psum += x;
-            pf[j][4 * sub + r] = (T)x;
-          }
-        l[j] = l[j] * alpha + psum;
-        // the running maximum settles after the first chunks: skip the 4*NDT multiplies when no lane rescales
-        if (__ballot(alpha != 1.f)) {
-#pragma unroll
-          for (int i = 0; i < NDT; i++) acc[j][i] *= alpha;
         }
-      }
+      };
+      // chunks every token of the wave sees completely (all but the one or two at the causal edge)
+      // take the path without per-element visibility tests
+      if (32 * ch >= wave_lo_max && 32 * ch + 32 <= wave_hi_min) softmax(std::false_type{});
+      else softmax(std::true_type{});
 #pragma unroll
       for (int dt = 0; dt < NDT; dt++) {
         const v8 vt = tr_frag<T, LD>(v_s[buf], 16 * dt, li, lg);
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[j][dt] = E::mfma16(vt, pf[j], acc[j][dt]);
+        for (int j = 0; j < TPW; j++) acc[j][dt] = E::mfma16(vt, pf[j], acc[j][dt]);
       }
     }
   };
@@ -241,11 +258,10 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
     }
   }
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int pos = ti.i0 + 4 * wave + j;
+  for (int j = 0; j < TPW; j++) {
+    const int pos = ti.i0 + TPW * wave + j;
     float lt = l[j];
-    lt += __shfl_xor(lt, 16);
-    lt += __shfl_xor(lt, 32);
+    lt = column_sum(lt);
     if (pos < ti.lq && has_head) {
       const float inv = lt > 0.f ? 1.f / lt : 0.f;
       T* op = (T*)p.o + (long long)(ti.s0q + pos) * p.osn + (long long)hh * p.osh + 4 * lg;
@@ -256,7 +272,7 @@ __global__ __launch_bounds__(256) void cmp_fwd_kernel(CmpParams p) {
         for (int r = 0; r < 4; r++) out[r] = (T)(acc[j][dt][r] * inv);
         st8(op + 16 * dt, out);
       }
-      if (lg == 0) p.lse[(long long)hh * p.total_q + ti.s0q + pos] = lt > 0.f ? m[j] + fast_log2(lt) : -INFINITY;
+      if (lg == 0) p.lse[(long long)hh * p.total_q + ti.s0q + pos] = lt > 0.f ? m[j] * p.qk_scale + fast_log2(lt) : -INFINITY;
     }
   }
 }
@@ -464,8 +480,7 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
 #pragma unroll
               for (int r = 0; r < 4; r++) x += fast_exp2(s[r] * p.qk_scale - l2[j][r]);
             }
-            x += __shfl_xor(x, 16);
-            x += __shfl_xor(x, 32);
+            x = column_sum(x);
             if (lg == 0) my_sc[j * SC_W + pad + 16 * sub + li] = x;
           }
         }
@@ -591,7 +606,7 @@ template <typename T, int D>
 static int run_cmp(CmpArgs& a) {
   const int64_t slots = n_tile_slots(a.Tq, a.B);
   if (a.what == 0) {
-    cmp_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
+    cmp_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)(a.Hkv * a.p.GT)), 64 * (16 / FWD_TPW), 0, a.stream>>>(a.p);
   } else if (a.what == 1) {
     const size_t dyn = ((size_t)16 * a.sp.nb_cap + 4 * 4 * SC_W) * 4;
     if (dyn > 64 * 1024) {

@@ -82,8 +82,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
       s[r] = x;
       mw = fmaxf(mw, x);
     }
-    mw = fmaxf(mw, __shfl_xor(mw, 16));
-    mw = fmaxf(mw, __shfl_xor(mw, 32));
+    mw = column_max(mw);
     float lw = 0.f;
     v8 pf = zero16<v8>();
 #pragma unroll
@@ -92,8 +91,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
       lw += x;
       pf[r] = (T)x;
     }
-    lw += __shfl_xor(lw, 16);
-    lw += __shfl_xor(lw, 32);
+    lw = column_sum(lw);
     if (lg == 0) { m_s[wave][li] = mw; l_s[wave][li] = lw; }
     __syncthreads();  // v_s staged, m_s/l_s visible
     float m = fmaxf(fmaxf(m_s[0][li], m_s[1][li]), fmaxf(m_s[2][li], m_s[3][li]));

@@ -60,6 +60,35 @@ template <typename V> __device__ __forceinline__ void st8(void* p, V v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// Reductions over the four lanes {l, l^16, l^32, l^48} that share one MFMA column, as VALU
+// lane swaps (v_permlane32_swap / v_permlane16_swap) instead of LDS-crossbar shuffles. After a
+// swap of x with itself the two results hold, for every lane, its own half and the partner's.
+// The halves are copied into scalars before the float reinterpretation: reinterpreting a
+// vector element in place reads element 0 for every index.
+typedef unsigned nsa_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void lane_halves32(float x, float& a, float& b) {
+  const unsigned u = __float_as_uint(x);
+  const nsa_u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  a = __uint_as_float(r0); b = __uint_as_float(r1);
+}
+__device__ __forceinline__ void lane_halves16(float x, float& a, float& b) {
+  const unsigned u = __float_as_uint(x);
+  const nsa_u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  a = __uint_as_float(r0); b = __uint_as_float(r1);
+}
+__device__ __forceinline__ float column_max(float x) {
+  float a, b;
+  lane_halves32(x, a, b); x = fmaxf(a, b);
+  lane_halves16(x, a, b); return fmaxf(a, b);
+}
+__device__ __forceinline__ float column_sum(float x) {
+  float a, b;
+  lane_halves32(x, a, b); x = a + b;
+  lane_halves16(x, a, b); return a + b;
+}
+
 // Index of the sequence that holds global token t: largest b with cu[b] <= t.
 __device__ __forceinline__ int find_sequence(const int32_t* __restrict__ cu, int batch, int t) {
   int lo = 0, hi = batch;  // invariant: cu[lo] <= t < cu[hi]

@@ -102,8 +102,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
           s[nt][r] = x;
           mloc = fmaxf(mloc, x);
         }
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+      mloc = column_max(mloc);
       const float m_new = fmaxf(m, mloc);  // finite: key0 <= pos is always visible
       const float alpha = fast_exp2(m - m_new);
       m = m_new;
@@ -133,8 +132,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
     }
   }
   }
-  lsum += __shfl_xor(lsum, 16);
-  lsum += __shfl_xor(lsum, 32);
+  lsum = column_sum(lsum);
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
   if (has_head) {
     T* op = (T*)p.o + (long long)t * p.osn + (long long)(h * p.G + hq) * p.osh + 4 * lg;
