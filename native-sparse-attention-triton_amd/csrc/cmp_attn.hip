@@ -82,7 +82,7 @@ struct Stager {
       ok |= (unsigned)(key < lk) << u;
     }
   }
-  __device__ __forceinline__ void stash(T (*ta)[D + 8], T (*tb)[D + 8], int tid) {
+  __device__ __forceinline__ void stash(T (*ta)[lds_pitch(D)], T (*tb)[lds_pitch(D)], int tid) {
 #pragma unroll
     for (int u = 0; u < PPT; u++) {
       const int pc = tid + u * NT;
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams 
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8, TPW = FWD_TPW, NT = 64 * (16 / TPW);
+  constexpr int NK = D / 32, NDT = D / 16, LD = lds_pitch(D), TPW = FWD_TPW, NT = 64 * (16 / TPW);
   __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
   __shared__ __attribute__((aligned(16))) T v_s[2][32][LD];
   TileInfo ti;
@@ -169,93 +169,117 @@ __global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams 
   }
   const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
   const T* vb = (const T*)p.v + (long long)ti.k0 * p.vsn + (long long)h * p.vsh;
-  // two register stages with fixed roles (the loop is unrolled by two): chunk ch+2 is requested while
-  // chunk ch is being consumed, so a full chunk of compute hides each load
-  Stager<T, D, 2, NT> stg0, stg1;
-  if (n_chunks > ch0) {
-    stg0.fetch(kb, p.ksn, vb, p.vsn, ch0, ti.lk, tid);
-    stg0.stash(k_s[0], v_s[0], tid);
-    stg1.fetch(kb, p.ksn, vb, p.vsn, min(ch0 + 1, n_chunks - 1), ti.lk, tid);
-  }
-  __syncthreads();
-  auto compute = [&](const int ch, const int buf) {
-    if (32 * ch < wave_hi && 32 * ch + 32 > wave_lo) {
-      f32x4 s[TPW][2];
+  // Software pipeline over the 32-key chunks.  Iteration ch holds, in one basic block, the MFMAs of
+  // P(ch-1) V(ch-1) and of S(ch+1) = K(ch+1) Q^T together with the softmax arithmetic of S(ch): the
+  // matrix pipe and the vector ALU work on different chunks, so neither waits for the other.  K and V
+  // tiles therefore live in LDS for different spans: iteration ch reads K(ch+1) and V(ch-1) and
+  // writes K(ch+2) and V(ch) (fetched into registers one iteration earlier) into the other parity.
+  Stager<T, D, 1, NT> sk, sv;
+  auto qk = [&](const int buf, f32x4 (&s)[TPW][2]) {
 #pragma unroll
-      for (int sub = 0; sub < 2; sub++) {
-        v8 kf[NK];
+    for (int sub = 0; sub < 2; sub++) {
+      v8 kf[NK];
 #pragma unroll
-        for (int kk = 0; kk < NK; kk++) kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
+      for (int kk = 0; kk < NK; kk++) kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
 #pragma unroll
-        for (int j = 0; j < TPW; j++) {
-          f32x4 c = {0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < TPW; j++) {
+        f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int kk = 0; kk < NK; kk++) c = E::mfma16(kf[kk], qf[j][kk], c);
-          s[j][sub] = c;
-        }
-      }
-      v8 pf[TPW];
-      // Running maxima are kept in raw score units with a finite floor, so a token that sees nothing
-      // yet needs no special case: exp2(-inf - finite) is 0 and the floor minus itself gives alpha 1.
-      auto softmax = [&](auto masked) {
-#pragma unroll
-        for (int j = 0; j < TPW; j++) {
-          float mloc = M_FLOOR;
-#pragma unroll
-          for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-              if (decltype(masked)::value) {
-                const int c = 32 * ch + 16 * sub + 4 * lg + r;
-                if (!(c >= lo[j] && c < hi[j])) s[j][sub][r] = -INFINITY;
-              }
-              mloc = fmaxf(mloc, s[j][sub][r]);
-            }
-          mloc = column_max(mloc);
-          const float m_new = fmaxf(m[j], mloc);
-          const float alpha = fast_exp2((m[j] - m_new) * p.qk_scale);
-          const float mb = m_new * p.qk_scale;
-          m[j] = m_new;
-          float psum = 0.f;
-#pragma unroll
-          for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-              const float x = fast_exp2(__builtin_fmaf(s[j][sub][r], p.qk_scale, -mb));
-              psum += x;
-              pf[j][4 * sub + r] = (T)x;
-            }
-          l[j] = l[j] * alpha + psum;
-          // the running maximum settles after the first chunks: skip the 4*NDT multiplies when no lane rescales
-          if (__ballot(alpha != 1.f)) {
-#pragma unroll
-            for (int i = 0; i < NDT; i++) acc[j][i] *= alpha;
-          }
-        }
-      };
-      // chunks every token of the wave sees completely (all but the one or two at the causal edge)
-      // take the path without per-element visibility tests
-      if (32 * ch >= wave_lo_max && 32 * ch + 32 <= wave_hi_min) softmax(std::false_type{});
-      else softmax(std::true_type{});
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++) {
-        const v8 vt = tr_frag<T, LD>(v_s[buf], 16 * dt, li, lg);
-#pragma unroll
-        for (int j = 0; j < TPW; j++) acc[j][dt] = E::mfma16(vt, pf[j], acc[j][dt]);
+        for (int kk = 0; kk < NK; kk++) c = E::mfma16(kf[kk], qf[j][kk], c);
+        s[j][sub] = c;
       }
     }
   };
-  for (int ch = ch0; ch < n_chunks; ch += 2) {
-    stg0.fetch(kb, p.ksn, vb, p.vsn, min(ch + 2, n_chunks - 1), ti.lk, tid);
-    compute(ch, 0);
-    if (ch + 1 < n_chunks) stg1.stash(k_s[1], v_s[1], tid);
+  auto pv = [&](const int buf, const v8 (&pf)[TPW]) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++) {
+      const v8 vt = tr_frag<T, LD>(v_s[buf], 16 * dt, li, lg);
+#pragma unroll
+      for (int j = 0; j < TPW; j++) acc[j][dt] = E::mfma16(vt, pf[j], acc[j][dt]);
+    }
+  };
+  // Running maxima are kept in raw score units with a finite floor, so a token that sees nothing yet
+  // needs no special case: exp2(-inf - finite) is 0 and the floor minus itself gives alpha 1.
+  float alpha[TPW];
+  auto softmax = [&](auto masked, const int ch, f32x4 (&s)[TPW][2], v8 (&pf)[TPW]) {
+#pragma unroll
+    for (int j = 0; j < TPW; j++) {
+      float mloc = M_FLOOR;
+#pragma unroll
+      for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          if (decltype(masked)::value) {
+            const int c = 32 * ch + 16 * sub + 4 * lg + r;
+            if (!(c >= lo[j] && c < hi[j])) s[j][sub][r] = -INFINITY;
+          }
+          mloc = fmaxf(mloc, s[j][sub][r]);
+        }
+      mloc = column_max(mloc);
+      const float m_new = fmaxf(m[j], mloc);
+      alpha[j] = fast_exp2((m[j] - m_new) * p.qk_scale);
+      const float mb = m_new * p.qk_scale;
+      m[j] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float x = fast_exp2(__builtin_fmaf(s[j][sub][r], p.qk_scale, -mb));
+          psum += x;
+          pf[j][4 * sub + r] = (T)x;
+        }
+      l[j] = l[j] * alpha[j] + psum;
+    }
+  };
+  if (n_chunks > ch0) {
+    const int last = n_chunks - 1;
+    f32x4 s_cur[TPW][2], s_nxt[TPW][2];
+    v8 pf[TPW];
+#pragma unroll
+    for (int j = 0; j < TPW; j++) pf[j] = zero16<v8>();
+    // P = 0 meets the not yet written V tile of the other parity in the first iteration: clear it
+    for (int i = tid; i < 32 * LD / 8; i += NT) reinterpret_cast<uint4*>(&v_s[(ch0 + 1) & 1][0][0])[i] = uint4{0u, 0u, 0u, 0u};
+    sk.fetch(kb, p.ksn, kb, p.ksn, ch0, ti.lk, tid);
+    sk.stash(k_s[ch0 & 1], k_s[ch0 & 1], tid);
+    sk.fetch(kb, p.ksn, kb, p.ksn, min(ch0 + 1, last), ti.lk, tid);
+    sk.stash(k_s[(ch0 + 1) & 1], k_s[(ch0 + 1) & 1], tid);
+    sk.fetch(kb, p.ksn, kb, p.ksn, min(ch0 + 2, last), ti.lk, tid);
+    sv.fetch(vb, p.vsn, vb, p.vsn, ch0, ti.lk, tid);
     __syncthreads();
-    if (ch + 1 < n_chunks) {
-      stg1.fetch(kb, p.ksn, vb, p.vsn, min(ch + 3, n_chunks - 1), ti.lk, tid);
-      compute(ch + 1, 1);
-      if (ch + 2 < n_chunks) stg0.stash(k_s[0], v_s[0], tid);
+    qk(ch0 & 1, s_cur);
+    __syncthreads();
+    for (int ch = ch0; ch < n_chunks; ch++) {
+      const int par = ch & 1;
+      sk.stash(k_s[par], k_s[par], tid);
+      sv.stash(v_s[par], v_s[par], tid);
+      sk.fetch(kb, p.ksn, kb, p.ksn, min(ch + 3, last), ti.lk, tid);
+      sv.fetch(vb, p.vsn, vb, p.vsn, min(ch + 1, last), ti.lk, tid);
+      // chunks every token of the wave sees completely (all but the one or two at the causal edge) take
+      // the path without per-element visibility tests
+      if (32 * ch >= wave_lo_max && 32 * ch + 32 <= wave_hi_min) {
+        pv(par ^ 1, pf);
+        qk(par ^ 1, s_nxt);
+        softmax(std::false_type{}, ch, s_cur, pf);
+      } else {
+        pv(par ^ 1, pf);
+        qk(par ^ 1, s_nxt);
+        softmax(std::true_type{}, ch, s_cur, pf);
+      }
+      // the running maximum settles after the first chunks: skip the multiplies when no lane rescales
+#pragma unroll
+      for (int j = 0; j < TPW; j++)
+        if (__ballot(alpha[j] != 1.f)) {
+#pragma unroll
+          for (int i = 0; i < NDT; i++) acc[j][i] *= alpha[j];
+        }
+#pragma unroll
+      for (int j = 0; j < TPW; j++)
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) s_cur[j][sub] = s_nxt[j][sub];
       __syncthreads();
     }
+    pv(last & 1, pf);
   }
 #pragma unroll
   for (int j = 0; j < TPW; j++) {
@@ -283,7 +307,7 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8, TPW = 2;  // tokens per wave: 8-token tiles inside the 16-token slot
+  constexpr int NK = D / 32, NDT = D / 16, LD = lds_pitch(D), TPW = 2;  // tokens per wave: 8-token tiles inside the 16-token slot
   __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
   __shared__ __attribute__((aligned(16))) T v_s[2][32][LD];
   TileInfo ti;
@@ -411,7 +435,7 @@ template <typename T, int D>
 __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
-  constexpr int NK = D / 32, LD = D + 8;
+  constexpr int NK = D / 32, LD = lds_pitch(D);
   __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
   extern __shared__ float dyn[];
   float* bs_s = dyn;                           // [16][nb_cap] block scores of the tile's tokens

@@ -22,7 +22,7 @@ template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
-  constexpr int NK = D / 32, NDT = D / 16, LD = D + 8;
+  constexpr int NK = D / 32, NDT = D / 16, LD = lds_pitch(D);
   __shared__ __attribute__((aligned(16))) T v_s[4][16][LD];
   __shared__ float m_s[4][16], l_s[4][16];
   __shared__ float o_s[16][D + 1];

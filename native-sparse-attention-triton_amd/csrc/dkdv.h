@@ -71,7 +71,7 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
   constexpr int NW = dkdv_waves(BS);          // waves per workgroup
   constexpr int KT = NSUB / NW;               // 16-key tiles per wave
   constexpr int NT = NW * 64;
-  constexpr int LD = D + 8;                   // padded LDS row (elements)
+  constexpr int LD = lds_pitch(D);                   // padded LDS row (elements)
   __shared__ __attribute__((aligned(16))) T q_s[2][2][16][LD];
   __shared__ __attribute__((aligned(16))) T do_s[2][2][16][LD];
   __shared__ __attribute__((aligned(16))) float lse_s[2][32], delta_s[2][32];

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(LinParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NET = D / 16, LD = D + 8, PIECES = 32 * (D / 8), PPT = (PIECES + 255) / 256;
+  constexpr int NK = D / 32, NET = D / 16, LD = lds_pitch(D), PIECES = 32 * (D / 8), PPT = (PIECES + 255) / 256;
   __shared__ __attribute__((aligned(16))) T w_s[2][32][LD];
   const int h = blockIdx.y;
   const int b = slot_sequence(p.ycu, p.batch, blockIdx.x, 64);
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void lin_dw_kernel(LinParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NET = D / 16, LD = D + 8;
+  constexpr int NET = D / 16, LD = lds_pitch(D);
   constexpr int DTW = (D / 16 + 3) / 4;  // d tiles per wave
   __shared__ __attribute__((aligned(16))) T x_s[2][32][LD];
   __shared__ __attribute__((aligned(16))) T g_s[2][32][LD];

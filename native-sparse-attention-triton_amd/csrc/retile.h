@@ -28,7 +28,7 @@ __device__ __forceinline__ int seq_first_slot(const int32_t* __restrict__ cu, in
 template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256) void retile_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu, int batch,
                                                      long long stride_n, long long stride_h, int n_slots) {
-  __shared__ __attribute__((aligned(16))) T tile[32][D + 8];
+  __shared__ __attribute__((aligned(16))) T tile[32][lds_pitch(D)];
   const int slot = blockIdx.x, h = blockIdx.y;
   int lo = 0, hi = batch;
   while (hi - lo > 1) {
