@@ -20,6 +20,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wno-unused-value",
     # keep the compiler from forming packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # let MFMA accumulators live in ordinary VGPRs: accumulators that the vector ALU also touches
+    # (online-softmax rescale, epilogues) otherwise get copied to and from AGPRs around every MFMA group
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 

@@ -102,9 +102,6 @@ struct Stager {
   }
 };
 
-// floor of the running score maxima (raw q.k units): finite, so differences of maxima never form inf - inf
-#define M_FLOOR (-1e30f)
-
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 // fragment of X^T for 16 columns starting at d0 over the 32 staged rows, in the k-order of the

@@ -13,6 +13,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define NSA_LOG2E 1.4426950408889634f
+// floor of the running score maxima (raw q.k units): finite, so differences of maxima never form inf - inf
+#define M_FLOOR (-1e30f)
+// how far (in powers of two) a new maximum may exceed the reference maximum before online-softmax
+// accumulators are rescaled
+#define RESCALE_SLACK 8.f
 
 // Element-type traits: 8-wide register fragments and the 16x16x32 / 32x32x16 MFMA for that type.
 // Fragment layout (wave64): A is [16][32] with lane l holding row l%16, k = 8*(l/16)..+7;

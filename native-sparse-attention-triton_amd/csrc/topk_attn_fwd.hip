@@ -19,12 +19,14 @@ struct TopkFwdParams {
 };
 
 template <typename T, int D, int BS>
-__global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void topk_fwd_kernel(TopkFwdParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   constexpr int NK = D / 32, NDT = D / 16;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // the wave index is made a scalar so that everything derived from it (token, sequence, block ids,
+  // fragment addresses) is computed once per wave on the scalar unit
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, lg = lane >> 4;
   const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
   if (item >= p.n_items) return;
@@ -46,11 +48,12 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
   f32x4 acc[NDT];
 #pragma unroll
   for (int i = 0; i < NDT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, lsum = 0.f;
+  float m = M_FLOOR, lsum = 0.f;
 
   const int32_t* ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
-  const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
-  const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
+  const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D;  // wave-uniform; lanes add lane * 8
+  const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D;
+  const unsigned lane8 = lane * 8u;
 
   const int last_slot = (len - 1) >> 5;  // last slot of this sequence that exists in the copies
   // the row of block ids is read once, 64 entries at a time (lane e holds entry e); the valid
@@ -76,13 +79,13 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
         // sub-tiles wholly in the future are masked below; clamp them onto storage that exists
         const int st = min((key0 >> 4) + nt, 2 * last_slot + 1);
 #pragma unroll
-        for (int kk = 0; kk < NK; kk++) kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512);
+        for (int kk = 0; kk < NK; kk++) kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512 + lane8);
       }
 #pragma unroll
       for (int c = 0; c < NC; c++) {
         const int slot = min((key0 >> 5) + c, last_slot);
 #pragma unroll
-        for (int dt = 0; dt < NDT; dt++) vfr[c][dt] = ld16<v8>(vbase + (long long)slot * D * 32 + dt * 512);
+        for (int dt = 0; dt < NDT; dt++) vfr[c][dt] = ld16<v8>(vbase + (long long)slot * D * 32 + dt * 512 + lane8);
       }
       f32x4 s[NS];
 #pragma unroll
@@ -92,32 +95,44 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
         for (int kk = 0; kk < NK; kk++) c = E::mfma16(kfr[nt][kk], qf[kk], c);
         s[nt] = c;
       }
-      float mloc = -INFINITY;
+      // only the slice that holds the query's own position needs the causal test
+      if (key0 + 16 * NS - 1 > pos) {
+#pragma unroll
+        for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (key0 + 16 * nt + 4 * lg + r > pos) s[nt][r] = -INFINITY;
+      }
+      float mloc = M_FLOOR;
 #pragma unroll
       for (int nt = 0; nt < NS; nt++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int key = key0 + 16 * nt + 4 * lg + r;
-          const float x = key <= pos ? s[nt][r] * p.qk_scale : -INFINITY;
-          s[nt][r] = x;
-          mloc = fmaxf(mloc, x);
-        }
+        for (int r = 0; r < 4; r++) mloc = fmaxf(mloc, s[nt][r]);
       mloc = column_max(mloc);
-      const float m_new = fmaxf(m, mloc);  // finite: key0 <= pos is always visible
-      const float alpha = fast_exp2(m - m_new);
-      m = m_new;
+      // The reference maximum m (raw q.k units) only moves when a slice beats it by more than
+      // RESCALE_SLACK in the exponent: until then probabilities are formed against the old reference
+      // (at most 2^RESCALE_SLACK, exact in fp32 sums and within range of bf16/fp16), and the
+      // accumulator rescale, a multiply per accumulator register, is skipped.
+      const bool moved = (mloc - m) * p.qk_scale > RESCALE_SLACK;
+      if (__ballot(moved)) {
+        const float m_new = moved ? mloc : m;
+        const float alpha = fast_exp2((m - m_new) * p.qk_scale);
+        m = m_new;
+        lsum *= alpha;
+#pragma unroll
+        for (int i = 0; i < NDT; i++) acc[i] *= alpha;
+      }
+      const float mb = m * p.qk_scale;
       float psum = 0.f;
 #pragma unroll
       for (int nt = 0; nt < NS; nt++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float x = fast_exp2(s[nt][r] - m_new);
+          const float x = fast_exp2(__builtin_fmaf(s[nt][r], p.qk_scale, -mb));
           s[nt][r] = x;
           psum += x;
         }
-      lsum = lsum * alpha + psum;
-#pragma unroll
-      for (int i = 0; i < NDT; i++) acc[i] *= alpha;
+      lsum += psum;
 #pragma unroll
       for (int c = 0; c < NC; c++) {
         v8 pf;  // probabilities of masked keys are exactly 0, the clamped V data they meet is finite
@@ -143,7 +158,7 @@ __global__ __launch_bounds__(256) void topk_fwd_kernel(TopkFwdParams p) {
       for (int r = 0; r < 4; r++) out[r] = (T)(acc[dt][r] * inv);
       st8(op + 16 * dt, out);
     }
-    if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + t] = lsum > 0.f ? m + fast_log2(lsum) : -INFINITY;
+    if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + t] = lsum > 0.f ? m * p.qk_scale + fast_log2(lsum) : -INFINITY;
   }
 }
 
