@@ -426,7 +426,8 @@ struct SelParams {
   long long qsn, qsh, ksn, ksh, osh, osn, osk;
   float qk_scale;
 };
-static constexpr int SC_W = 32 + 16;  // per-token score strip: carry (<=16) + one 32-key chunk
+
+constexpr int SEL_LOCAL = 16;  // candidates a lane keeps in registers during selection (64 * SEL_LOCAL blocks)
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
@@ -436,25 +437,23 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
   __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
   extern __shared__ float dyn[];
   float* bs_s = dyn;                           // [16][nb_cap] block scores of the tile's tokens
-  float* sc_s = dyn + 16 * p.nb_cap;           // [4 waves][4 tokens][SC_W]
   TileInfo ti;
   if (!locate_tile(p.cu_q, p.cu_k, p.batch, blockIdx.x, ti)) return;
   const int h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
-  const int a = p.ks / p.st, rr = p.bs / p.st, pad = a - 1, n_taps = a + rr - 1;
-  const int nbl = 32 / rr;  // blocks completed by one 32-key chunk
+  const int a = p.ks / p.st, rr = p.bs / p.st;  // keys per kernel window and per selection block
   for (int i = tid; i < 16 * p.nb_cap; i += 256) bs_s[i] = 0.f;
   int lim[4];
-  int wave_lim = 0;
+  int wave_lim = 0, wave_lim_min = 1 << 30;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     lim[j] = visible_keys(ti.i0 + 4 * wave + j, ti.lq, ti.lk, p.ks, p.st);
     wave_lim = max(wave_lim, lim[j]);
+    wave_lim_min = min(wave_lim_min, lim[j]);
   }
   const int tile_last = min(ti.i0 + 15, ti.lq - 1);
   const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
   const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
-  float* my_sc = sc_s + wave * 4 * SC_W;
   Stager<T, D, 1> stg;
   __syncthreads();
   for (int gt = 0; gt < p.GT; gt++) {
@@ -475,7 +474,7 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
         l2[j][r] = (hr < p.G && pos < ti.lq) ? p.lse[(long long)(h * p.G + hr) * p.total_q + t] : INFINITY;
       }
     }
-    for (int i = lane; i < 4 * SC_W; i += 64) my_sc[i] = 0.f;  // carry of "chunk -1"
+    float xprev = 0.f;  // scores of the 16 keys before the current ones (none before key 0)
     if (n_chunks > 0) {
       stg.fetch(kb, p.ksn, kb, p.ksn, 0, ti.lk, tid);
       stg.stash(k_s[0], k_s[0], tid);
@@ -485,44 +484,49 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
       const int buf = ch & 1;
       if (ch + 1 < n_chunks) stg.fetch(kb, p.ksn, kb, p.ksn, ch + 1, ti.lk, tid);
       if (32 * ch < wave_lim) {
+        // all 8 score tiles of the chunk first (independent MFMA chains), then the exponentials in bulk
+        f32x4 s[2][4];
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
           v8 kf[NK];
 #pragma unroll
           for (int kk = 0; kk < NK; kk++) kf[kk] = ld16<v8>(&k_s[buf][16 * sub + li][32 * kk + 8 * lg]);
-          const int c = 32 * ch + 16 * sub + li;  // this lane's key (column)
 #pragma unroll
           for (int j = 0; j < 4; j++) {
-            f32x4 s = {0.f, 0.f, 0.f, 0.f};
+            f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < NK; kk++) s = E::mfma16(qf[j][kk], kf[kk], s);  // rows = heads 4*lg+r
+            for (int kk = 0; kk < NK; kk++) c = E::mfma16(qf[j][kk], kf[kk], c);  // rows = heads 4*lg+r
+            s[sub][j] = c;
+          }
+        }
+        const bool edge = 32 * ch + 32 > wave_lim_min;  // some token of the wave does not see the whole chunk
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+          const int c = 32 * ch + 16 * sub + li;  // this lane's key (column)
+          float xs = 0.f;                         // lane group lg keeps the scores of the wave's token lg
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
             float x = 0.f;
-            if (c < lim[j]) {
 #pragma unroll
-              for (int r = 0; r < 4; r++) x += fast_exp2(s[r] * p.qk_scale - l2[j][r]);
-            }
+            for (int r = 0; r < 4; r++) x += fast_exp2(__builtin_fmaf(s[sub][j][r], p.qk_scale, -l2[j][r]));
+            if (edge) x = c < lim[j] ? x : 0.f;
             x = column_sum(x);
-            if (lg == 0) my_sc[j * SC_W + pad + 16 * sub + li] = x;
+            xs = lg == j ? x : xs;
           }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int i = lane; i < 4 * nbl; i += 64) {
-          const int j = i / nbl, lb = i % nbl;
-          const int blk = (32 * ch) / rr + lb;
-          float v = 0.f;
-          for (int o = 0; o < n_taps; o++) {
-            const int w = min(min(o, n_taps - 1 - o), min(a - 1, rr - 1)) + 1;
-            v += (float)w * my_sc[j * SC_W + lb * rr + o];
+          // Overlap weights = box(a) convolved with box(rr): first the sum over the a keys that end at
+          // each key (reaching into the previous 16 keys, kept in xprev), then the sum over the rr keys
+          // of a block, both as lane exchanges inside the 16 lanes of a token.
+          float z = xs;
+          for (int u = 1; u < a; u++) {
+            const float same = __shfl(xs, lane - u), before = __shfl(xprev, lane + 16 - u);
+            z += li >= u ? same : before;
           }
-          if (blk < p.full_blocks && blk < p.nb_cap) bs_s[(4 * wave + j) * p.nb_cap + blk] += v;
+          xprev = xs;
+          for (int mk = 1; mk < rr && mk < 16; mk <<= 1) z += __shfl_xor(z, mk);
+          const int blk = c / rr;
+          if ((li & (min(rr, 16) - 1)) == 0 && blk < p.full_blocks && blk < p.nb_cap)
+            atomicAdd(&bs_s[(4 * wave + lg) * p.nb_cap + blk], z);  // LDS add without return: nothing waits for it
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        float carry = 0.f;
-        if (lane < 4 * pad) carry = my_sc[(lane / pad) * SC_W + 32 + lane % pad];
-        __builtin_amdgcn_wave_barrier();
-        if (lane < 4 * pad) my_sc[(lane / pad) * SC_W + lane % pad] = carry;
       }
       if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], k_s[buf ^ 1], tid);
       __syncthreads();
@@ -545,23 +549,51 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
       for (int i = lane; i < p.k_out; i += 64) out[(long long)i * p.osk] = i < nb ? i : -1;
       continue;
     }
-    for (int round = 0; round < n_pick; round++) {
+    // Every lane owns the blocks lane, lane + 64, ... and remembers the best of them; a round is one
+    // wave-wide maximum over those, after which only the owner of the winner updates its best.
+    if (nb <= 64 * SEL_LOCAL) {
+      // the lane's candidates fit in registers: no LDS traffic inside the rounds
+      float cand[SEL_LOCAL];
+#pragma unroll
+      for (int i = 0; i < SEL_LOCAL; i++) cand[i] = lane + 64 * i < nb ? row[lane + 64 * i] : -3.f;
       float bv = -1.f;
       int bi = 0x7fffffff;
-      for (int blk = lane; blk < nb; blk += 64) {
-        const float v = row[blk];
-        if (v > bv) { bv = v; bi = blk; }
-      }
 #pragma unroll
-      for (int sft = 32; sft > 0; sft >>= 1) {
-        const float ov = __shfl_xor(bv, sft);
-        const int oi = __shfl_xor(bi, sft);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      for (int i = 0; i < SEL_LOCAL; i++)
+        if (cand[i] > bv) { bv = cand[i]; bi = lane + 64 * i; }
+      for (int round = 0; round < n_pick; round++) {
+        const int win = candidate_index(wave_max_i64(candidate_key(bv, bi)));
+        if (bi == win) {
+          row[win] = -2.f;  // taken
+          bv = -1.f; bi = 0x7fffffff;
+#pragma unroll
+          for (int i = 0; i < SEL_LOCAL; i++) {
+            if (lane + 64 * i == win) cand[i] = -2.f;
+            if (cand[i] > bv) { bv = cand[i]; bi = lane + 64 * i; }
+          }
+        }
       }
-      if (lane == 0) row[bi] = -2.f;  // taken
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+    } else {
+      float bv;
+      int bi;
+      auto rescan = [&]() {
+        bv = -1.f; bi = 0x7fffffff;
+        for (int blk = lane; blk < nb; blk += 64) {
+          const float v = row[blk];
+          if (v > bv) { bv = v; bi = blk; }
+        }
+      };
+      rescan();
+      for (int round = 0; round < n_pick; round++) {
+        const int win = candidate_index(wave_max_i64(candidate_key(bv, bi)));
+        if (bi == win) {
+          row[win] = -2.f;  // taken
+          rescan();
+        }
+      }
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     int base = 0;
     for (int blk0 = 0; blk0 < nb; blk0 += 64) {
       const int blk = blk0 + lane;
@@ -629,7 +661,7 @@ static int run_cmp(CmpArgs& a) {
   if (a.what == 0) {
     cmp_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)(a.Hkv * a.p.GT)), 64 * (16 / FWD_TPW), 0, a.stream>>>(a.p);
   } else if (a.what == 1) {
-    const size_t dyn = ((size_t)16 * a.sp.nb_cap + 4 * 4 * SC_W) * 4;
+    const size_t dyn = (size_t)16 * a.sp.nb_cap * 4;
     if (dyn > 64 * 1024) {
       if (hipFuncSetAttribute((const void*)cmp_select_kernel<T, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
         return NSA_ERR_UNSUPPORTED;
@@ -717,10 +749,11 @@ extern "C" int nsa_cmp_attn_select(const void* q, const void* k, const float* ls
   if (!lse || !out_topk_idx || k_out <= 0 || max_seqlen_q <= 0) return NSA_ERR_BAD_ARG;
   if (kernel_size % kernel_stride != 0 || block_size % kernel_size != 0) return NSA_ERR_BAD_ARG;
   const int64_t rr = block_size / kernel_stride, pad = kernel_size / kernel_stride - 1;
-  if (rr > 32 || 32 % rr != 0 || pad > 16) return NSA_ERR_UNSUPPORTED;
+  // the lane-exchange fold of key scores into block scores needs a power-of-two block and a window of at most 16 keys
+  if ((rr & (rr - 1)) != 0 || pad > 15) return NSA_ERR_UNSUPPORTED;
   const int64_t nb = (max_seqlen_q + block_size - 1) / block_size;
   if (k_out > nb) return NSA_ERR_BAD_ARG;
-  if (((size_t)16 * nb + 4 * 4 * SC_W) * 4 > 140 * 1024) return NSA_ERR_UNSUPPORTED;  // block-score strip must fit LDS
+  if ((size_t)16 * nb * 4 > 140 * 1024) return NSA_ERR_UNSUPPORTED;  // block scores of a 16-token tile must fit LDS
   SelParams& s = a.sp;
   s.q = q; s.k = k; s.lse = lse; s.cu_q = cu_seqlens_q; s.cu_k = cu_seqlens_k; s.out = out_topk_idx;
   s.total_q = (int)total_q; s.batch = (int)batch; s.Hkv = (int)num_kv_heads; s.G = a.p.G; s.GT = a.p.GT; s.ks = (int)kernel_size;

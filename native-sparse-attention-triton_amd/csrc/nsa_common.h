@@ -100,6 +100,44 @@ __device__ __forceinline__ float column_sum(float x) {
   lane_halves16(x, a, b); return a + b;
 }
 
+// Wave-wide maximum of a signed 64-bit key, returned to every lane: four DPP steps inside each row of
+// 16 lanes (pair, quad, half-row mirror, row mirror), then the two lane swaps across rows.
+template <int CTRL> __device__ __forceinline__ long long dpp_exchange64(long long k) {
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(unsigned)(unsigned long long)k, CTRL, 0xf, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(k >> 32), CTRL, 0xf, 0xf, false);
+  return ((long long)hi << 32) | (unsigned)lo;
+}
+__device__ __forceinline__ long long wave_max_i64(long long k) {
+  long long o;
+  o = dpp_exchange64<0xB1>(k); k = o > k ? o : k;   // quad_perm [1,0,3,2]
+  o = dpp_exchange64<0x4E>(k); k = o > k ? o : k;   // quad_perm [2,3,0,1]
+  o = dpp_exchange64<0x141>(k); k = o > k ? o : k;  // row_half_mirror
+  o = dpp_exchange64<0x140>(k); k = o > k ? o : k;  // row_mirror
+  {
+    const unsigned lo = (unsigned)(unsigned long long)k, hi = (unsigned)((unsigned long long)k >> 32);
+    const nsa_u32x2 a = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
+    const nsa_u32x2 b = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
+    const unsigned a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1];
+    const long long x = ((long long)(int)b0 << 32) | a0, y = ((long long)(int)b1 << 32) | a1;
+    k = x > y ? x : y;
+  }
+  {
+    const unsigned lo = (unsigned)(unsigned long long)k, hi = (unsigned)((unsigned long long)k >> 32);
+    const nsa_u32x2 a = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+    const nsa_u32x2 b = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+    const unsigned a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1];
+    const long long x = ((long long)(int)b0 << 32) | a0, y = ((long long)(int)b1 << 32) | a1;
+    k = x > y ? x : y;
+  }
+  return k;
+}
+// Sort key of a (score, index) candidate: larger score first, smaller index on ties.  Scores here are
+// non-negative (or +inf), whose bit patterns order like the numbers; negative markers sort below.
+__device__ __forceinline__ long long candidate_key(float score, int index) {
+  return ((long long)__float_as_int(score) << 32) | (unsigned)(0x7fffffff - index);
+}
+__device__ __forceinline__ int candidate_index(long long key) { return 0x7fffffff - (int)(unsigned)(unsigned long long)key; }
+
 // Index of the sequence that holds global token t: largest b with cu[b] <= t.
 __device__ __forceinline__ int find_sequence(const int32_t* __restrict__ cu, int batch, int t) {
   int lo = 0, hi = batch;  // invariant: cu[lo] <= t < cu[hi]
