@@ -429,7 +429,15 @@ struct SelParams {
 
 constexpr int SEL_LOCAL = 16;  // candidates a lane keeps in registers during selection (64 * SEL_LOCAL blocks)
 
-template <typename T, int D>
+// sum over the A keys that end at each lane's key: lanes below in this row, then the tail of the previous 16 keys
+template <int U, int A> __device__ __forceinline__ float window_sum(float xs, float xprev) {
+  if constexpr (U >= A) return 0.f;
+  else return dpp_f32<0x110 + U>(xs) + dpp_f32<0x100 + 16 - U>(xprev) + window_sum<U + 1, A>(xs, xprev);
+}
+
+// A, RR: keys per kernel window and per selection block when they are the compile-time pair handled
+// with DPP lane moves (A = 0: any power-of-two pair, through run-time lane shuffles).
+template <typename T, int D, int A, int RR>
 __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
@@ -440,8 +448,8 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
   TileInfo ti;
   if (!locate_tile(p.cu_q, p.cu_k, p.batch, blockIdx.x, ti)) return;
   const int h = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
-  const int a = p.ks / p.st, rr = p.bs / p.st;  // keys per kernel window and per selection block
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), li = lane & 15, lg = lane >> 4;
+  const int a = A ? A : p.ks / p.st, rr = A ? RR : p.bs / p.st;  // keys per kernel window and per selection block
   for (int i = tid; i < 16 * p.nb_cap; i += 256) bs_s[i] = 0.f;
   int lim[4];
   int wave_lim = 0, wave_lim_min = 1 << 30;
@@ -503,26 +511,33 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
           const int c = 32 * ch + 16 * sub + li;  // this lane's key (column)
-          float xs = 0.f;                         // lane group lg keeps the scores of the wave's token lg
+          float x[4];
 #pragma unroll
           for (int j = 0; j < 4; j++) {
-            float x = 0.f;
+            x[j] = 0.f;
 #pragma unroll
-            for (int r = 0; r < 4; r++) x += fast_exp2(__builtin_fmaf(s[sub][j][r], p.qk_scale, -l2[j][r]));
-            if (edge) x = c < lim[j] ? x : 0.f;
-            x = column_sum(x);
-            xs = lg == j ? x : xs;
+            for (int r = 0; r < 4; r++) x[j] += fast_exp2(__builtin_fmaf(s[sub][j][r], p.qk_scale, -l2[j][r]));
+            if (edge) x[j] = c < lim[j] ? x[j] : 0.f;
           }
+          const float xs = column_sum_scatter4(x[0], x[1], x[2], x[3]);  // lane group lg: token lg, summed over all heads
           // Overlap weights = box(a) convolved with box(rr): first the sum over the a keys that end at
           // each key (reaching into the previous 16 keys, kept in xprev), then the sum over the rr keys
           // of a block, both as lane exchanges inside the 16 lanes of a token.
           float z = xs;
-          for (int u = 1; u < a; u++) {
-            const float same = __shfl(xs, lane - u), before = __shfl(xprev, lane + 16 - u);
-            z += li >= u ? same : before;
+          if constexpr (A != 0) {
+            z += window_sum<1, A>(xs, xprev);
+            if constexpr (RR >= 2) z += dpp_f32<0xB1>(z);
+            if constexpr (RR >= 4) z += dpp_f32<0x4E>(z);
+            if constexpr (RR >= 8) z += dpp_f32<0x141>(z);
+            if constexpr (RR >= 16) z += dpp_f32<0x140>(z);
+          } else {
+            for (int u = 1; u < a; u++) {
+              const float same = __shfl(xs, lane - u), before = __shfl(xprev, lane + 16 - u);
+              z += li >= u ? same : before;
+            }
+            for (int mk = 1; mk < rr && mk < 16; mk <<= 1) z += __shfl_xor(z, mk);
           }
           xprev = xs;
-          for (int mk = 1; mk < rr && mk < 16; mk <<= 1) z += __shfl_xor(z, mk);
           const int blk = c / rr;
           if ((li & (min(rr, 16) - 1)) == 0 && blk < p.full_blocks && blk < p.nb_cap)
             atomicAdd(&bs_s[(4 * wave + lg) * p.nb_cap + blk], z);  // LDS add without return: nothing waits for it
@@ -662,11 +677,14 @@ static int run_cmp(CmpArgs& a) {
     cmp_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)(a.Hkv * a.p.GT)), 64 * (16 / FWD_TPW), 0, a.stream>>>(a.p);
   } else if (a.what == 1) {
     const size_t dyn = (size_t)16 * a.sp.nb_cap * 4;
+    // kernel 32 / stride 16 / block 64 (the published configuration) gets the compile-time fold
+    const bool usual = a.sp.ks == 2 * a.sp.st && a.sp.bs == 4 * a.sp.st;
+    const void* fn = usual ? (const void*)cmp_select_kernel<T, D, 2, 4> : (const void*)cmp_select_kernel<T, D, 0, 0>;
     if (dyn > 64 * 1024) {
-      if (hipFuncSetAttribute((const void*)cmp_select_kernel<T, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
-        return NSA_ERR_UNSUPPORTED;
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess) return NSA_ERR_UNSUPPORTED;
     }
-    cmp_select_kernel<T, D><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
+    if (usual) cmp_select_kernel<T, D, 2, 4><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
+    else cmp_select_kernel<T, D, 0, 0><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
   } else {
     const CmpBwdLayout L = cmp_bwd_layout(a.Tq, a.Tk, a.B, a.Hq, a.Hkv, D);
     float* delta = (float*)(a.ws + L.delta);

@@ -100,6 +100,26 @@ __device__ __forceinline__ float column_sum(float x) {
   lane_halves16(x, a, b); return a + b;
 }
 
+// Sums over the four lanes of a column for four values at once: on return the lanes of group g (lanes
+// 16g..16g+15) hold the column sums of x_g.  Three swaps and three adds instead of four column_sum calls.
+__device__ __forceinline__ float column_sum_scatter4(float x0, float x1, float x2, float x3) {
+  const nsa_u32x2 p = __builtin_amdgcn_permlane32_swap(__float_as_uint(x0), __float_as_uint(x2), false, false);
+  const nsa_u32x2 q = __builtin_amdgcn_permlane32_swap(__float_as_uint(x1), __float_as_uint(x3), false, false);
+  const unsigned p0 = p[0], p1 = p[1], q0 = q[0], q1 = q[1];
+  const float y02 = __uint_as_float(p0) + __uint_as_float(p1);  // lower half: x0 over both halves, upper half: x2
+  const float y13 = __uint_as_float(q0) + __uint_as_float(q1);
+  const nsa_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(y02), __float_as_uint(y13), false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  return __uint_as_float(r0) + __uint_as_float(r1);
+}
+
+// Value of another lane of the same 16-lane row by a DPP control word (0x110 + n: from n lanes below,
+// 0x100 + n: from n lanes above, both 0 where that lane is outside the row; 0xB1 / 0x4E: partner in a
+// pair / quad; 0x141 / 0x140: mirror within 8 / 16 lanes).
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+
 // Wave-wide maximum of a signed 64-bit key, returned to every lane: four DPP steps inside each row of
 // 16 lanes (pair, quad, half-row mirror, row mirror), then the two lane swaps across rows.
 template <int CTRL> __device__ __forceinline__ long long dpp_exchange64(long long k) {
