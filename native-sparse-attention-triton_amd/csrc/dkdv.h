@@ -20,13 +20,6 @@ static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
 // of 32 keys need > 256 registers each (one wave per SIMD) and measured 17% slower than four.
 constexpr int dkdv_waves(int bs) { return bs >= 64 ? 4 : bs / 16; }
 
-// LDS row that holds head hd of a staged 16-head row group.  The transposed reads of one
-// half-wave address the rows of heads {4*lg + j : lg in {0,1}, j < 4} (the other half-wave those of
-// lg in {2,3}); with the 272-byte row pitch these must be even (odd) rows to fall on 32 different
-// 8-byte bank pairs.  The plain 16-byte fragment reads touch all 16 rows and stay conflict-free
-// under any permutation.
-__device__ __forceinline__ int lds_row_of_head(int hd) { return ((((hd >> 2) & 1) * 4 + (hd & 3)) << 1) | (hd >> 3); }
-
 // chunk_off = exclusive scan of ceil((seg_end - seg_begin)/CHUNK_TOKENS) over segments (single workgroup).
 static __global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* __restrict__ seg_begin, const int32_t* __restrict__ seg_end, int n_seg,
                                                           int32_t* __restrict__ chunk_off) {
@@ -177,8 +170,8 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
         uint4 a = sg.qd[u], b2 = sg.dd[u];
         a.x &= m; a.y &= m; a.z &= m; a.w &= m;
         b2.x &= m; b2.y &= m; b2.z &= m; b2.w &= m;
-        *reinterpret_cast<uint4*>(&q_s[buf][rg][lds_row_of_head(hd)][8 * c]) = a;
-        *reinterpret_cast<uint4*>(&do_s[buf][rg][lds_row_of_head(hd)][8 * c]) = b2;
+        *reinterpret_cast<uint4*>(&q_s[buf][rg][hd][8 * c]) = a;
+        *reinterpret_cast<uint4*>(&do_s[buf][rg][hd][8 * c]) = b2;
       }
     }
     if (tid < 32) {
@@ -202,8 +195,8 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < NK; kk++) {
-          v8 qa = ld16<v8>(&q_s[buf][tk][lds_row_of_head(li)][32 * kk + 8 * lg]);
-          v8 da = ld16<v8>(&do_s[buf][tk][lds_row_of_head(li)][32 * kk + 8 * lg]);
+          v8 qa = ld16<v8>(&q_s[buf][tk][li][32 * kk + 8 * lg]);
+          v8 da = ld16<v8>(&do_s[buf][tk][li][32 * kk + 8 * lg]);
           s = E::mfma16(qa, kf[j][kk], s);
           dp = E::mfma16(da, vf[j][kk], dp);
         }
@@ -231,8 +224,8 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
       s16x8 qt, dot;
 #pragma unroll
       for (int tk = 0; tk < 2; tk++) {
-        const T* qa = &q_s[buf][tk][lds_row_of_head(4 * lg + (li >> 2))][16 * dt + 4 * (li & 3)];
-        const T* da = &do_s[buf][tk][lds_row_of_head(4 * lg + (li >> 2))][16 * dt + 4 * (li & 3)];
+        const T* qa = &q_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+        const T* da = &do_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
         s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(qa));
         s16x4 c = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(da));
 #pragma unroll
