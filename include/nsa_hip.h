@@ -158,15 +158,22 @@ int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, const void* o,
                      int64_t kernel_stride, const int64_t* strides, float sm_scale, int dtype, void* workspace,
                      size_t workspace_bytes, void* stream);
 
-/* ---- sliding-window prefill (forward only) ---------------------------------------------------
+/* ---- sliding-window attention ----------------------------------------------------------------
  * Stands in for flash_attn_varlen_func(..., causal=True, window_size=(window_size, -1)) as called from
- * native_sparse_attention/infer/inference_func.py:180-190 (a third-party kernel in the reference):
- * position i attends to keys j of its sequence with i - window_size <= j <= i.
- * strides (HOST int64[8]): q(n,h) k(n,h) v(n,h) o(n,h); lse fp32 [Hq,T] base-2.
+ * native_sparse_attention/infer/inference_func.py:180-190 (prefill) and
+ * native_sparse_attention/module/native_sparse_attention.py:213-223 (training; a third-party kernel
+ * in the reference): position i attends to keys j of its sequence with i - window_size <= j <= i.
+ * Forward strides (HOST int64[8]): q(n,h) k(n,h) v(n,h) o(n,h); lse fp32 [Hq,T] base-2.
+ * Backward strides (HOST int64[16]): q k v o dout dq dk dv, (n,h) each; workspace 256-byte aligned.
  */
 int nsa_window_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
                         int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                         int64_t window_size, const int64_t* strides, float sm_scale, int dtype, void* stream);
+size_t nsa_window_attn_bwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim);
+int nsa_window_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse, void* dq, void* dk,
+                        void* dv, const int32_t* cu_seqlens, int64_t total_len, int64_t batch, int64_t num_q_heads,
+                        int64_t num_kv_heads, int64_t head_dim, int64_t window_size, const int64_t* strides, float sm_scale,
+                        int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- decode (one query per sequence over KV-cache slabs [B, slab_len, Hkv, D]) ---------------
  * strides: HOST int64 array: q(b,h) k(b,n,h) v(b,n,h) o(b,h) [+ idx(h,b,k) for the entry points

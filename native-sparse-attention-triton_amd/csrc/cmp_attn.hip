@@ -317,14 +317,15 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
   const bool has_head = hq < p.G;
   const int hh = h * p.G + (has_head ? hq : 0);
   v8 qf[TPW][NK], dof[TPW][NK];
-  int lim[TPW];
+  int lo[TPW], hi[TPW];
   float l2[TPW], dl[TPW];
-  int wave_lim = 0;
+  int wave_lo = 1 << 30, wave_hi = 0;
 #pragma unroll
   for (int j = 0; j < TPW; j++) {
     const int pos = ti.i0 + TPW * wave + j;
-    lim[j] = visible_keys(pos, ti.lq, ti.lk, p.ks, p.st);
-    wave_lim = max(wave_lim, lim[j]);
+    visible_range(pos, ti.lq, ti.lk, p.ks, p.st, p.window, lo[j], hi[j]);
+    wave_hi = max(wave_hi, hi[j]);
+    if (hi[j] > 0) wave_lo = min(wave_lo, lo[j]);
     const bool live = has_head && pos < ti.lq;
     const long long t = ti.s0q + (pos < ti.lq ? pos : 0);
     const T* qp = (const T*)p.q + t * p.qsn + (long long)hh * p.qsh + 8 * lg;
@@ -337,8 +338,11 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
     l2[j] = live ? p.lse[(long long)hh * p.total_q + t] : INFINITY;
     dl[j] = live ? p.delta[(long long)hh * p.total_q + t] : 0.f;
   }
-  const int tile_last = min(ti.i0 + 7, ti.lq - 1);
-  const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
+  int tile_lo, tile_hi, unused;
+  visible_range(min(ti.i0 + 7, ti.lq - 1), ti.lq, ti.lk, p.ks, p.st, p.window, unused, tile_hi);
+  visible_range(ti.i0, ti.lq, ti.lk, p.ks, p.st, p.window, tile_lo, unused);
+  const int ch0 = tile_lo / 32;                 // the first token of the tile reaches furthest back
+  const int n_chunks = (tile_hi + 31) / 32;
   f32x4 acc[TPW][NDT];
 #pragma unroll
   for (int j = 0; j < TPW; j++)
@@ -349,14 +353,14 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
   // two register stages with fixed roles (the loop is unrolled by two): chunk ch+2 is requested while
   // chunk ch is being consumed, so a full chunk of compute hides each load
   Stager<T, D, 2> stg0, stg1;
-  if (n_chunks > 0) {
-    stg0.fetch(kb, p.ksn, vb, p.vsn, 0, ti.lk, tid);
+  if (n_chunks > ch0) {
+    stg0.fetch(kb, p.ksn, vb, p.vsn, ch0, ti.lk, tid);
     stg0.stash(k_s[0], v_s[0], tid);
-    stg1.fetch(kb, p.ksn, vb, p.vsn, min(0 + 1, n_chunks - 1), ti.lk, tid);
+    stg1.fetch(kb, p.ksn, vb, p.vsn, min(ch0 + 1, n_chunks - 1), ti.lk, tid);
   }
   __syncthreads();
   auto compute = [&](const int ch, const int buf) {
-    if (32 * ch < wave_lim) {
+    if (32 * ch < wave_hi && 32 * ch + 32 > wave_lo) {
       v8 dsf[TPW];
 #pragma unroll
       for (int sub = 0; sub < 2; sub++) {
@@ -377,7 +381,7 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             const int c = 32 * ch + 16 * sub + 4 * lg + r;
-            const float pr = c < lim[j] ? fast_exp2(s[r] * p.qk_scale - l2[j]) : 0.f;
+            const float pr = (c >= lo[j] && c < hi[j]) ? fast_exp2(s[r] * p.qk_scale - l2[j]) : 0.f;
             dsf[j][4 * sub + r] = (T)(pr * (dp[r] - dl[j]) * p.sm_scale);
           }
         }
@@ -390,7 +394,7 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
       }
     }
   };
-  for (int ch = 0; ch < n_chunks; ch += 2) {
+  for (int ch = ch0; ch < n_chunks; ch += 2) {
     stg0.fetch(kb, p.ksn, vb, p.vsn, min(ch + 2, n_chunks - 1), ti.lk, tid);
     compute(ch, 0);
     if (ch + 1 < n_chunks) stg1.stash(k_s[1], v_s[1], tid);
@@ -626,7 +630,7 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
 // dK/dV segments: blocks of 64 compressed keys per (head, sequence); their queries are the
 // contiguous range from the first position that sees the block's first key to the sequence end
 __global__ void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cu_k, int batch, int Hkv, int ks, int st,
-                                    int max_blocks, int32_t* __restrict__ cu_blk, int32_t* __restrict__ seg_begin, int32_t* __restrict__ seg_end) {
+                                    int window, int max_blocks, int32_t* __restrict__ cu_blk, int32_t* __restrict__ seg_begin, int32_t* __restrict__ seg_end) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   int acc = 0;
   cu_blk[0] = 0;
@@ -638,7 +642,8 @@ __global__ void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int3
       for (int g = cu_blk[b]; g < cu_blk[b + 1]; g++) {
         const int first_pos = (g - cu_blk[b]) * 64 * st + ks - 1;
         seg_begin[h * max_blocks + g] = cu_q[b] + min(first_pos, lq);
-        seg_end[h * max_blocks + g] = cu_q[b] + lq;
+        // window mode (ordinary keys): the block's last key 64*g' + 63 is seen up to position 64*g' + 63 + window
+        seg_end[h * max_blocks + g] = cu_q[b] + (window < 0 ? lq : (int)min((long long)lq, (long long)(g - cu_blk[b]) * 64 + 64 + window));
       }
     }
   }
@@ -694,14 +699,14 @@ static int run_cmp(CmpArgs& a) {
     int32_t* chunk_off = (int32_t*)(a.ws + L.chunk_off);
     const int n_seg = (int)(a.Hkv * L.max_blocks);
     launch_delta<T, D>((const T*)a.o_in, (const T*)a.p.dout, delta, a.Tq, a.Hq, a.p.osn, a.p.osh, a.p.dsn, a.p.dsh, a.stream);
-    cmp_segments_kernel<<<1, 64, 0, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
+    cmp_segments_kernel<<<1, 64, 0, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
     chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off);
     DkdvParams d;
     d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
     d.cu_blk = cu_blk; d.seg_begin = seg_begin; d.seg_end = seg_end; d.chunk_off = chunk_off; d.queries = nullptr;
     d.partial = (float*)(a.ws + L.partial);
     d.total_len = (int)a.Tq; d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;
-    d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st;
+    d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st; d.window = a.p.window;
     d.qsn = (int)a.p.qsn; d.qsh = (int)a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = (int)a.p.dsn; d.dsh = (int)a.p.dsh;
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
     if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
@@ -809,8 +814,8 @@ extern "C" int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, con
   return cmp_dispatch(a, head_dim, dtype);
 }
 
-// Causal sliding-window (or, with a window >= the longest sequence, plain causal) varlen attention,
-// forward only: the same tile kernel with the visibility rule "j in [i - window, i]".
+// Causal sliding-window (or, with a window >= the longest sequence, plain causal) varlen attention:
+// the same tile kernels with the visibility rule "j in [i - window, i]".
 extern "C" int nsa_window_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
                                    int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                                    int64_t window_size, const int64_t* strides, float sm_scale, int dtype, void* stream) {
@@ -821,5 +826,30 @@ extern "C" int nsa_window_attn_fwd(const void* q, const void* k, const void* v, 
   a.p.o = o; a.p.lse = lse; a.p.osn = strides[6]; a.p.osh = strides[7];
   a.p.window = (int)(window_size > (1 << 30) ? (1 << 30) : window_size);
   a.what = 0;
+  return cmp_dispatch(a, head_dim, dtype);
+}
+
+extern "C" size_t nsa_window_attn_bwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim) {
+  return cmp_bwd_layout(total_len, total_len, batch, num_q_heads, num_kv_heads, head_dim).total;
+}
+
+extern "C" int nsa_window_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse, void* dq,
+                                   void* dk, void* dv, const int32_t* cu_seqlens, int64_t total_len, int64_t batch, int64_t num_q_heads,
+                                   int64_t num_kv_heads, int64_t head_dim, int64_t window_size, const int64_t* strides, float sm_scale,
+                                   int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, v, cu_seqlens, cu_seqlens, total_len, total_len, batch, num_q_heads, num_kv_heads, 1, 1, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!v || !o || !dout || !lse || !dq || !dk || !dv || !workspace || window_size < 0) return NSA_ERR_BAD_ARG;
+  for (int i = 6; i < 10; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
+  for (int i = 10; i < 16; i++) if (strides[i] % 4 != 0) return NSA_ERR_UNSUPPORTED;
+  if (((uintptr_t)o | (uintptr_t)dout) % 16 != 0 || ((uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) % 8 != 0 || (uintptr_t)workspace % 256 != 0) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_window_attn_bwd_workspace_bytes(total_len, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
+  a.o_in = o; a.p.dout = dout; a.p.lse = (float*)lse; a.p.dq = dq; a.dk = dk; a.dv = dv;
+  a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
+  a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
+  a.p.window = (int)(window_size > (1 << 30) ? (1 << 30) : window_size);
+  a.ws = (char*)workspace;
+  a.what = 2;
   return cmp_dispatch(a, head_dim, dtype);
 }

@@ -292,7 +292,7 @@ static int run_bwd(const BwdArgs& a) {
     p.partial = (float*)(ws + L.partial);
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
     p.qsn = (int)a.qsn; p.qsh = (int)a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = (int)a.dsn; p.dsh = (int)a.dsh;
-    p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1;
+    p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1; p.window = -1;
     constexpr int NT = 64 * dkdv_waves(BS);
     if (GT == 1) dkdv_kernel<T, D, BS, false, true><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
     else dkdv_kernel<T, D, BS, false, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
