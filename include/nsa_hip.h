@@ -175,6 +175,18 @@ int nsa_window_attn_bwd(const void* q, const void* k, const void* v, const void*
                         int64_t num_kv_heads, int64_t head_dim, int64_t window_size, const int64_t* strides, float sm_scale,
                         int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- rotary position embedding ---------------------------------------------------------------
+ * Replaces RotaryEmbedding.forward of native_sparse_attention/module/rope.py:199-209 (cos/sin tables
+ * :120-152, per-sequence positions :154-197): x, out [n_rows, H, D] (strides in elements, multiples of 8),
+ * inv_freq fp32 [D/2] on the device.  step == 0: row n is token (n - cu_seqlens[b]) of sequence b and is
+ * rotated for position (n - cu_seqlens[b]) * stride.  step > 0 (decode): n_rows == batch, row b is rotated
+ * for position (cu_seqlens[b+1] - cu_seqlens[b] + step - 1) * stride.  inverse != 0 applies the transposed
+ * rotation (the gradient of the forward call).
+ */
+int nsa_rope(const void* x, void* out, const float* inv_freq, const int32_t* cu_seqlens, int64_t n_rows, int64_t batch,
+             int64_t num_heads, int64_t head_dim, int64_t x_stride_n, int64_t x_stride_h, int64_t o_stride_n, int64_t o_stride_h,
+             int64_t step, int64_t stride, float attention_scaling, int inverse, int dtype, void* stream);
+
 /* ---- decode (one query per sequence over KV-cache slabs [B, slab_len, Hkv, D]) ---------------
  * strides: HOST int64 array: q(b,h) k(b,n,h) v(b,n,h) o(b,h) [+ idx(h,b,k) for the entry points
  * that read or write topk ids] = 10 or 13 values.  q/k/v strides must be multiples of 8.

@@ -1,0 +1,86 @@
+// Rotary position embedding over varlen rows, x [N, H, D] -> out [N, H, D]:
+//   out[..., :D/2] = x1 * cos - x2 * sin,  out[..., D/2:] = x2 * cos + x1 * sin,  angle = position * inv_freq[i].
+// One workgroup per row: the first D/2 threads evaluate cos/sin of the row's position once (fp32, full
+// range reduction: angles reach 1e5 rad), every head then reuses them from LDS.  cos/sin and each product
+// are rounded to the element type before the next operation, as element-wise bf16/fp16 tensor arithmetic
+// does, so results match a framework-level x * cos + rotate_half(x) * sin.  HBM-bound: one read and one
+// write of x.
+#include "nsa_common.h"
+
+struct RopeParams {
+  const void* x; void* out; const float* inv_freq; const int32_t* cu;
+  int n_rows, batch, H, step, stride;
+  long long xsn, xsh, osn, osh;
+  float scaling;
+  int inverse;
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
+  using v8 = typename Elem<T>::v8;
+  constexpr int HALF = D / 2, VEC = HALF / 8;  // 8-element pieces per half row
+  __shared__ float cos_s[HALF], sin_s[HALF];
+  const int n = blockIdx.x;
+  int pos;
+  if (p.step == 0) {  // prefill: row n is token n - cu[b] of its sequence
+    const int b = find_sequence(p.cu, p.batch, n);
+    pos = (n - p.cu[b]) * p.stride;
+  } else {            // decode: one row per sequence, `step` tokens after its prompt
+    pos = (p.cu[n + 1] - p.cu[n] + p.step - 1) * p.stride;
+  }
+  if (threadIdx.x < HALF) {
+    const float ang = (float)pos * p.inv_freq[threadIdx.x];
+    const float c = (float)(T)(cosf(ang) * p.scaling), s = (float)(T)(sinf(ang) * p.scaling);
+    cos_s[threadIdx.x] = c;
+    sin_s[threadIdx.x] = p.inverse ? -s : s;
+  }
+  __syncthreads();
+  const T* xr = (const T*)p.x + (long long)n * p.xsn;
+  T* orow = (T*)p.out + (long long)n * p.osn;
+  for (int i = threadIdx.x; i < p.H * VEC; i += 256) {
+    const int h = i / VEC, c8 = (i % VEC) * 8;
+    const v8 x1 = ld16<v8>(xr + (long long)h * p.xsh + c8), x2 = ld16<v8>(xr + (long long)h * p.xsh + HALF + c8);
+    v8 o1, o2;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float c = cos_s[c8 + e], s = sin_s[c8 + e];
+      const float a1 = (float)x1[e], a2 = (float)x2[e];
+      const T x1c = (T)(a1 * c), x2s = (T)(a2 * s), x2c = (T)(a2 * c), x1s = (T)(a1 * s);
+      o1[e] = (T)((float)x1c - (float)x2s);
+      o2[e] = (T)((float)x2c + (float)x1s);
+    }
+    st16(orow + (long long)h * p.osh + c8, o1);
+    st16(orow + (long long)h * p.osh + HALF + c8, o2);
+  }
+}
+
+template <typename T>
+static int rope_dispatch(const RopeParams& p, int d, hipStream_t s) {
+  switch (d) {
+    case 32: rope_kernel<T, 32><<<p.n_rows, 256, 0, s>>>(p); break;
+    case 64: rope_kernel<T, 64><<<p.n_rows, 256, 0, s>>>(p); break;
+    case 96: rope_kernel<T, 96><<<p.n_rows, 256, 0, s>>>(p); break;
+    case 128: rope_kernel<T, 128><<<p.n_rows, 256, 0, s>>>(p); break;
+    default: return NSA_ERR_UNSUPPORTED;
+  }
+  return nsa_check_launch();
+}
+
+extern "C" int nsa_rope(const void* x, void* out, const float* inv_freq, const int32_t* cu_seqlens, int64_t n_rows, int64_t batch,
+                        int64_t num_heads, int64_t head_dim, int64_t x_stride_n, int64_t x_stride_h, int64_t o_stride_n,
+                        int64_t o_stride_h, int64_t step, int64_t stride, float attention_scaling, int inverse, int dtype,
+                        void* stream) {
+  if (!x || !out || !inv_freq || !cu_seqlens) return NSA_ERR_BAD_ARG;
+  if (n_rows < 0 || batch <= 0 || num_heads <= 0 || step < 0 || stride <= 0 || n_rows >= (1ll << 31)) return NSA_ERR_BAD_ARG;
+  if (step > 0 && n_rows != batch) return NSA_ERR_BAD_ARG;
+  if ((x_stride_n | x_stride_h | o_stride_n | o_stride_h) % 8 != 0 || ((uintptr_t)x | (uintptr_t)out) % 16 != 0) return NSA_ERR_UNSUPPORTED;
+  if (n_rows == 0) return NSA_OK;
+  RopeParams p;
+  p.x = x; p.out = out; p.inv_freq = inv_freq; p.cu = cu_seqlens;
+  p.n_rows = (int)n_rows; p.batch = (int)batch; p.H = (int)num_heads; p.step = (int)step; p.stride = (int)stride;
+  p.xsn = x_stride_n; p.xsh = x_stride_h; p.osn = o_stride_n; p.osh = o_stride_h;
+  p.scaling = attention_scaling; p.inverse = inverse;
+  if (dtype == NSA_BF16) return rope_dispatch<__bf16>(p, (int)head_dim, (hipStream_t)stream);
+  if (dtype == NSA_FP16) return rope_dispatch<_Float16>(p, (int)head_dim, (hipStream_t)stream);
+  return NSA_ERR_UNSUPPORTED;
+}

@@ -1,0 +1,95 @@
+"""Rotary embedding: the closed-form inverse frequencies against the library routine the reference calls
+(CPU), and the HIP kernel against an element-wise restatement of the reference's forward (GPU)."""
+import pytest
+import torch
+
+from native_sparse_attention.module.rope import RopeConfig, RotaryEmbedding, compute_inv_freq
+from native_sparse_attention.testing import cu_from_lens
+
+
+def test_inv_freq_matches_transformers_llama3():
+    transformers = pytest.importorskip("transformers")
+    from transformers.modeling_rope_utils import ROPE_INIT_FUNCTIONS
+    for d, theta in [(128, 500000.0), (64, 10000.0)]:
+        cfg = RopeConfig(head_dim=d, rope_theta=theta)
+        try:
+            lib_cfg = transformers.LlamaConfig(hidden_size=d, num_attention_heads=1, head_dim=d, max_position_embeddings=cfg.max_position_embeddings,
+                                               rope_parameters=dict(cfg.rope_scaling, rope_theta=theta))
+            want, scale = ROPE_INIT_FUNCTIONS["llama3"](lib_cfg, "cpu")
+        except (TypeError, AttributeError, KeyError) as e:  # another transformers generation: different config protocol
+            pytest.skip("installed transformers does not take this config: %r" % (e,))
+        got, got_scale = compute_inv_freq(cfg, "cpu")
+        assert torch.equal(got, want) and got_scale == scale == 1.0
+
+
+def test_inv_freq_default_and_bands():
+    cfg = RopeConfig(head_dim=64, rope_theta=10000.0, rope_scaling=None)
+    inv, _ = compute_inv_freq(cfg, "cpu")
+    assert torch.allclose(inv, 10000.0 ** (-torch.arange(0, 64, 2).float() / 64))
+    # llama3: short wavelengths untouched, long ones divided by the factor, monotone in between
+    cfg = RopeConfig()
+    base = 1.0 / (cfg.rope_theta ** (torch.arange(0, 128, 2).float() / 128))
+    inv, _ = compute_inv_freq(cfg, "cpu")
+    wl = 2 * torch.pi / base
+    assert torch.equal(inv[wl < 8192 / 4], base[wl < 8192 / 4])
+    assert torch.allclose(inv[wl > 8192], base[wl > 8192] / 8)
+    assert (inv[1:] < inv[:-1]).all()
+
+
+def _reference_forward(x, inv_freq, positions):
+    """rope.py:120-152,199-209 restated: cos/sin in fp32, cast to x.dtype, then x*cos + rotate_half(x)*sin
+    in x.dtype arithmetic."""
+    freqs = positions.float()[:, None] * inv_freq.float()[None, :]
+    cos = torch.cat([freqs.cos(), freqs.cos()], -1).to(x.dtype)[:, None, :]
+    sin = torch.cat([freqs.sin(), freqs.sin()], -1).to(x.dtype)[:, None, :]
+    half = x.shape[-1] // 2
+    rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return x * cos + rot * sin
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("lens,H,d,stride,dtype", [
+    ([100, 257, 31], 8, 128, 1, torch.bfloat16),
+    ([63, 447, 511], 4, 128, 16, torch.bfloat16),     # compressed keys: positions i * kernel_stride
+    ([300], 3, 64, 1, torch.float16),
+    ([40000], 1, 32, 3, torch.bfloat16),              # angles beyond 1e5 rad
+])
+def test_prefill_rotation_and_gradient(device, lens, H, d, stride, dtype):
+    g = torch.Generator(device=device).manual_seed(0)
+    cu = cu_from_lens(lens, device)
+    rope = RotaryEmbedding(RopeConfig(head_dim=d), device=device)
+    x = torch.randn(int(cu[-1]), H, d, generator=g, device=device).to(dtype)
+    pos = torch.cat([torch.arange(L, device=device) * stride for L in lens])
+    x1 = x.clone().requires_grad_()
+    y = rope(x1, cu, stride=stride)
+    want = _reference_forward(x, rope.inv_freq, pos)
+    # the same roundings on both sides; cos/sin of the two libraries may differ in the last bit, which moves a
+    # result by at most one unit in the last place of the element type
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    err = (y.float() - want.float()).abs()
+    assert (err <= ulp * want.float().abs().clamp(min=1.0)).all()
+    assert (y == want).float().mean() > 0.98
+    # gradient = the transposed rotation (checked against autograd of an fp32 statement)
+    dy = torch.randn(y.shape, generator=g, device=device).to(dtype)
+    y.backward(dy)
+    xf = x.float().requires_grad_()
+    freqs = pos.float()[:, None] * rope.inv_freq[None, :]
+    cos = torch.cat([freqs.cos(), freqs.cos()], -1)[:, None, :]
+    sin = torch.cat([freqs.sin(), freqs.sin()], -1)[:, None, :]
+    (xf * cos + torch.cat((-xf[..., d // 2:], xf[..., :d // 2]), -1) * sin).backward(dy.float())
+    assert (x1.grad.float() - xf.grad).abs().max() < 4e-2
+    assert (x1.grad.float() - xf.grad).abs().mean() < 4e-3
+
+
+@pytest.mark.gpu
+def test_decode_positions(device):
+    g = torch.Generator(device=device).manual_seed(1)
+    lens, H, d = [130, 47, 300], 8, 128
+    cu = cu_from_lens(lens, device)
+    rope = RotaryEmbedding(RopeConfig(head_dim=d), device=device)
+    x = torch.randn(len(lens), H, d, generator=g, device=device).bfloat16()
+    for step, stride in [(1, 1), (7, 1), (3, 16)]:
+        pos = torch.tensor([(L + step - 1) * stride for L in lens], device=device)
+        y = rope(x, cu, step=step, stride=stride)
+        want = _reference_forward(x, rope.inv_freq, pos)
+        assert ((y.float() - want.float()).abs() <= 2.0 ** -7 * want.float().abs().clamp(min=1.0)).all()
