@@ -187,6 +187,42 @@ int nsa_rope(const void* x, void* out, const float* inv_freq, const int32_t* cu_
              int64_t num_heads, int64_t head_dim, int64_t x_stride_n, int64_t x_stride_h, int64_t o_stride_n, int64_t o_stride_h,
              int64_t step, int64_t stride, float attention_scaling, int inverse, int dtype, void* stream);
 
+/* ---- KV-cache slabs ----------------------------------------------------------------------------
+ * Device-side counterparts of NSACache.prepare_compress / update_kv
+ * (native_sparse_attention/module/kv_cache.py:233-302, 340-449) and of its slab fill kernel (:453-555).
+ * A slab is a contiguous [2 (key, value), max_batch, rows, Hkv, D] array of 2-byte elements with an int32
+ * length per sequence; lengths are read and written on the device only.  Token tensors are [n, Hkv, D]
+ * with element strides (n, h), multiples of 8, D contiguous.
+ *
+ * nsa_cache_fill (prefill): for every sequence b, rows row_begin[b] .. row_end[b]-1 of key/value (cu_src gives
+ *   the sequence of every source row) go to slab[:, b, 0..]; slab_len[b] = row_end[b] - row_begin[b].
+ * nsa_cache_stage_token (decode, before compression): a staging window that holds kernel_size rows is shifted
+ *   left by kernel_stride, then the new token [batch, Hkv, D] is appended and stage_len incremented.
+ * nsa_cache_commit_token (decode, after compression and rotary embedding): tokens[6] = HOST array of device
+ *   pointers {compressed k, v, full-length k, v, sliding k, v}, strides = HOST int64[12] (n, h) for each; the
+ *   compressed pair is appended where stage_len[b] == kernel_size, the full-length pair is appended, the
+ *   sliding pair is written at row sliding_len[b] % window_size; the three lengths are incremented.
+ */
+int nsa_cache_fill(const void* key, const void* value, const int32_t* cu_src, const int32_t* row_begin, const int32_t* row_end,
+                   void* slab, int32_t* slab_len, int64_t total_rows, int64_t batch, int64_t num_kv_heads, int64_t head_dim,
+                   int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h, int64_t max_batch,
+                   int64_t slab_rows, void* stream);
+int nsa_cache_stage_token(const void* key, const void* value, void* stage_slab, int32_t* stage_len, int64_t batch,
+                          int64_t num_kv_heads, int64_t head_dim, int64_t k_stride_b, int64_t k_stride_h, int64_t v_stride_b,
+                          int64_t v_stride_h, int64_t max_batch, int64_t kernel_size, int64_t kernel_stride, void* stream);
+int nsa_cache_commit_token(const void* const* tokens, const int64_t* strides, const int32_t* stage_len, void* compress_slab,
+                           int32_t* compress_len, void* sparse_slab, int32_t* sparse_len, void* sliding_slab, int32_t* sliding_len,
+                           int64_t batch, int64_t num_kv_heads, int64_t head_dim, int64_t max_batch, int64_t kernel_size,
+                           int64_t compress_rows, int64_t sparse_rows, int64_t window_size, void* stream);
+
+/* ---- gated sum of the three branches -----------------------------------------------------------
+ * out[n, h, :] = gate[n, h, 0] * branch0 + gate[n, h, 1] * branch1 + gate[n, h, 2] * branch2, rounded step by
+ * step like the tensor expression of native_sparse_attention/infer/nsa_inference.py:146-150.
+ * strides (HOST int64[11]): gate (n, h, k), branch0 (n, h), branch1 (n, h), branch2 (n, h), out (n, h).
+ */
+int nsa_gate_combine(const void* gate, const void* branch0, const void* branch1, const void* branch2, void* out, int64_t n_rows,
+                     int64_t num_q_heads, int64_t head_dim, const int64_t* strides, int dtype, void* stream);
+
 /* ---- decode (one query per sequence over KV-cache slabs [B, slab_len, Hkv, D]) ---------------
  * strides: HOST int64 array: q(b,h) k(b,n,h) v(b,n,h) o(b,h) [+ idx(h,b,k) for the entry points
  * that read or write topk ids] = 10 or 13 values.  q/k/v strides must be multiples of 8.

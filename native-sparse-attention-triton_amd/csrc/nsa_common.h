@@ -62,6 +62,17 @@ template <typename V> __device__ __forceinline__ void st8(void* p, V v) {
   *reinterpret_cast<uint2*>(p) = __builtin_bit_cast(uint2, v);
 }
 
+// x rounded to the 2-byte element type T and widened again.  The compiler treats float -> T -> float as
+// removable and then contracts the surrounding multiply/add into an FMA; kernels that must reproduce
+// element-wise 16-bit tensor arithmetic (every product and sum rounded) pass the 16 bits through an opaque
+// register move so that the rounding stays.
+template <typename T> __device__ __forceinline__ float rounded(float x) {
+  const T t = (T)x;
+  unsigned bits = __builtin_bit_cast(unsigned short, t);
+  asm volatile("" : "+v"(bits));
+  return (float)__builtin_bit_cast(T, (unsigned short)bits);
+}
+
 // Row pitch (in 2-byte elements) of LDS tiles whose rows hold D elements.  Measured on gfx950: both the
 // 16-byte row-fragment reads (16 lanes on 16 rows, same column) and the transposing 8-byte reads (4
 // rows per 16 lanes) run at full rate exactly when the pitch in bytes is an odd multiple of 32; a pitch

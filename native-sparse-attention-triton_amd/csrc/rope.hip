@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
   }
   if (threadIdx.x < HALF) {
     const float ang = (float)pos * p.inv_freq[threadIdx.x];
-    const float c = (float)(T)(cosf(ang) * p.scaling), s = (float)(T)(sinf(ang) * p.scaling);
+    const float c = rounded<T>(cosf(ang) * p.scaling), s = rounded<T>(sinf(ang) * p.scaling);
     cos_s[threadIdx.x] = c;
     sin_s[threadIdx.x] = p.inverse ? -s : s;
   }
@@ -45,9 +45,8 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
     for (int e = 0; e < 8; e++) {
       const float c = cos_s[c8 + e], s = sin_s[c8 + e];
       const float a1 = (float)x1[e], a2 = (float)x2[e];
-      const T x1c = (T)(a1 * c), x2s = (T)(a2 * s), x2c = (T)(a2 * c), x1s = (T)(a1 * s);
-      o1[e] = (T)((float)x1c - (float)x2s);
-      o2[e] = (T)((float)x2c + (float)x1s);
+      o1[e] = (T)(rounded<T>(a1 * c) - rounded<T>(a2 * s));
+      o2[e] = (T)(rounded<T>(a2 * c) + rounded<T>(a1 * s));
     }
     st16(orow + (long long)h * p.osh + c8, o1);
     st16(orow + (long long)h * p.osh + HALF + c8, o2);

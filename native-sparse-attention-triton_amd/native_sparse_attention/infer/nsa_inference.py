@@ -10,6 +10,7 @@ from typing import Callable, Optional, Tuple
 
 import torch
 
+from .. import _lib
 from ..ops import (
     compressed_attention,
     compressed_attention_decode,
@@ -18,7 +19,7 @@ from ..ops import (
     topk_sparse_attention_decode,
 )
 from ..ops.sliding_window import sliding_window_attention_varlen
-from ..ops.utils import get_compressed_seqlens
+from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
 
 
 def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, intra_block_pe, kernel_size, kernel_stride):
@@ -46,10 +47,13 @@ def compressed_attention_infer(cu_seqlens, step, query, key, value, cache, kerne
                                     int(seqlens.max()), int(comp_seqlens.max()), None, init_blocks, local_blocks)
     batch = cu_seqlens.shape[0] - 1
     seqlens = cu_seqlens[1:] - cu_seqlens[:-1] + step
-    rows = int(cache.compress_kv_len[:batch].max())
+    # slab rows that can hold a compressed token at this step, from the host-side length bound (the reference
+    # slices by compress_kv_len.max(), inference_func.py:127-135, which waits for the device)
+    max_seqlen = cache.max_seqlen(step)
+    rows = min(max((max_seqlen - kernel_size) // kernel_stride + 1, 0), cache.max_comp_length)
     return compressed_attention_decode(query, cache.compress_kv_cache[0, :batch, :rows], cache.compress_kv_cache[1, :batch, :rows],
                                        seqlens, cache.compress_kv_len[:batch], kernel_size, kernel_stride, block_size, topk,
-                                       init_blocks, local_blocks)
+                                       init_blocks, local_blocks, max_seqlen=max_seqlen)
 
 
 def topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size):
@@ -66,6 +70,21 @@ def sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, w
     batch = cu_seqlens.shape[0] - 1
     lens = torch.clamp(cache.sliding_kv_len[:batch], max=window_size)
     return flash_attention_decode(query, cache.sliding_kv_cache[0, :batch], cache.sliding_kv_cache[1, :batch], lens)
+
+
+def gate_combine(gate_value, branch0, branch1, branch2):
+    """gate_value[..., 0, None] * branch0 + gate_value[..., 1, None] * branch1 + gate_value[..., 2, None] * branch2
+    (nsa_inference.py:146-150 of the reference) in one kernel, bit-identical to that expression.  No autograd."""
+    assert gate_value.shape == branch0.shape[:2] + (3,) and branch0.shape == branch1.shape == branch2.shape
+    assert gate_value.dtype == branch0.dtype == branch1.dtype == branch2.dtype
+    a, b, c = (last_dim_contiguous(t) for t in (branch0, branch1, branch2))
+    out = torch.empty_like(a, memory_format=torch.contiguous_format)
+    strides = _lib.host_i64([gate_value.stride(0), gate_value.stride(1), gate_value.stride(2), a.stride(0), a.stride(1), b.stride(0),
+                             b.stride(1), c.stride(0), c.stride(1), out.stride(0), out.stride(1)])
+    rc = _lib.load().nsa_gate_combine(gate_value.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), out.data_ptr(), a.shape[0],
+                                      a.shape[1], a.shape[2], strides, _lib.dtype_code(a), _lib.stream_ptr(a))
+    _lib.check(rc, "nsa_gate_combine")
+    return out
 
 
 def nsa_infer(
@@ -103,7 +122,7 @@ def nsa_infer(
                                                    kernel_stride, topk, block_size, init_blocks, local_blocks)
     sparse_out = topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size)
     window_out = sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size)
-    out = gate_value[..., 0, None] * cmp_out + gate_value[..., 1, None] * sparse_out + gate_value[..., 2, None] * window_out
+    out = gate_combine(gate_value, cmp_out, sparse_out, window_out)
     if return_branches:
         return out, (cmp_out, sparse_out, window_out, topk_idx)
     return out

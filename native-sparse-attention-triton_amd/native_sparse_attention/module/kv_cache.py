@@ -12,31 +12,30 @@ Decode-step rules (kv_cache.py:274-302, 401-449): a sequence whose staging windo
 shifts it left by kernel_stride, then the new token is appended; after compression the candidate
 compressed token is committed only for sequences whose staging window is full again; the new
 token is appended to the sparse slab and written into the ring at sliding_kv_len % window_size.
+
+Every update is one HIP kernel that reads and writes the length vectors on the device, so a decode step
+never waits for the host.  The only host-side figure is `max_seqlen` (longest prompt, taken once at
+prefill, plus the decode step), which bounds slab views and fixes output shapes.
 """
+import ctypes
 from typing import Union
 
 import torch
 
-from ..ops.utils import get_compressed_seqlens
-
-
-def _fill_slab(slab: torch.Tensor, key: torch.Tensor, value: torch.Tensor, seq_start: torch.Tensor, seq_end: torch.Tensor):
-    """slab[0 or 1, b, :seq_end[b]-seq_start[b]] = key or value[seq_start[b]:seq_end[b]] for every sequence."""
-    starts, ends = seq_start.tolist(), seq_end.tolist()
-    for b, (s, e) in enumerate(zip(starts, ends)):
-        if e > s:
-            slab[0, b, : e - s] = key[s:e]
-            slab[1, b, : e - s] = value[s:e]
+from .. import _lib
+from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
 
 
 class NSACache:
     def __init__(self, max_batch_size: int, max_length: int, num_kv_heads: int, head_dim: int, kernel_size: int,
                  kernel_stride: int, window_size: int, dtype: torch.dtype, device: Union[str, torch.device] = "cuda"):
+        assert dtype in (torch.bfloat16, torch.float16) and head_dim % 8 == 0 and kernel_size % kernel_stride == 0
         self.max_batch_size, self.max_length = max_batch_size, max_length
         self.num_kv_heads, self.head_dim = num_kv_heads, head_dim
         self.kernel_size, self.kernel_stride, self.window_size = kernel_size, kernel_stride, window_size
         self.dtype, self.device = dtype, device
         self.max_comp_length = (max_length - kernel_size) // kernel_stride + 1
+        self.max_prompt_len = 0  # host copy of the longest prompt of the current batch (set at prefill)
 
         def slab(rows):
             return torch.zeros(2, max_batch_size, rows, num_kv_heads, head_dim, dtype=dtype, device=device)
@@ -50,67 +49,70 @@ class NSACache:
         self.sliding_kv_cache, self.sliding_kv_len = slab(window_size), lens()
 
     def reset(self):
-        for t in (self.sparse_kv_cache, self.sparse_kv_len, self.compress_kv_cache, self.compress_kv_len,
-                  self.before_compress_kv_cache, self.before_compress_kv_len, self.sliding_kv_cache, self.sliding_kv_len):
+        # slab contents need no clearing: rows beyond the lengths are never read
+        for t in (self.sparse_kv_len, self.compress_kv_len, self.before_compress_kv_len, self.sliding_kv_len):
             t.zero_()
+        self.max_prompt_len = 0
+
+    def max_seqlen(self, step: int) -> int:
+        """Upper bound, known on the host, of every sequence's length at decode step `step`."""
+        return self.max_prompt_len + step
+
+    def _fill(self, slab, slab_len, key, value, cu_src, begin, end):
+        key, value = last_dim_contiguous(key), last_dim_contiguous(value)
+        batch = cu_src.shape[0] - 1
+        rc = _lib.load().nsa_cache_fill(key.data_ptr(), value.data_ptr(), cu_src.data_ptr(), begin.data_ptr(), end.data_ptr(),
+                                        slab.data_ptr(), slab_len.data_ptr(), key.shape[0], batch, self.num_kv_heads, self.head_dim,
+                                        key.stride(0), key.stride(1), value.stride(0), value.stride(1), self.max_batch_size,
+                                        slab.shape[2], _lib.stream_ptr(slab))
+        _lib.check(rc, "nsa_cache_fill")
 
     # ---- before compression -------------------------------------------------------------------
     def prepare_compress(self, cu_seqlens: torch.Tensor, step: int, key: torch.Tensor, value: torch.Tensor):
         assert key.shape == value.shape and key.shape[1:] == (self.num_kv_heads, self.head_dim)
+        assert key.dtype == self.dtype and value.dtype == self.dtype
+        batch = cu_seqlens.shape[0] - 1
+        assert batch <= self.max_batch_size
         if step == 0:
-            batch = cu_seqlens.shape[0] - 1
             comp_seqlens, _ = get_compressed_seqlens(cu_seqlens, self.kernel_size, self.kernel_stride)
             # tokens after the start of the next (incomplete) window wait in the staging slab
-            seq_start = cu_seqlens[:-1] + comp_seqlens * self.kernel_stride
-            seq_end = cu_seqlens[1:]
-            _fill_slab(self.before_compress_kv_cache, key, value, seq_start, seq_end)
-            self.before_compress_kv_len[:batch] = seq_end - seq_start
+            begin = (cu_seqlens[:-1] + comp_seqlens * self.kernel_stride).contiguous()
+            self._fill(self.before_compress_kv_cache, self.before_compress_kv_len, key, value, cu_seqlens, begin, cu_seqlens[1:].contiguous())
         else:
-            batch = key.shape[0]
-            assert batch == cu_seqlens.shape[0] - 1
-            full = self.before_compress_kv_len[:batch] == self.kernel_size
-            if bool(full.any()):
-                idx = torch.nonzero(full).flatten()
-                keep = self.kernel_size - self.kernel_stride
-                self.before_compress_kv_cache[:, idx, :keep] = self.before_compress_kv_cache[:, idx, self.kernel_stride:].clone()
-                self.before_compress_kv_len[idx] -= self.kernel_stride
-            rows = torch.arange(batch, device=key.device)
-            at = self.before_compress_kv_len[:batch].long()
-            self.before_compress_kv_cache[0, rows, at] = key
-            self.before_compress_kv_cache[1, rows, at] = value
-            self.before_compress_kv_len[:batch] += 1
+            assert key.shape[0] == batch
+            key, value = last_dim_contiguous(key), last_dim_contiguous(value)
+            rc = _lib.load().nsa_cache_stage_token(key.data_ptr(), value.data_ptr(), self.before_compress_kv_cache.data_ptr(),
+                                                   self.before_compress_kv_len.data_ptr(), batch, self.num_kv_heads, self.head_dim,
+                                                   key.stride(0), key.stride(1), value.stride(0), value.stride(1),
+                                                   self.max_batch_size, self.kernel_size, self.kernel_stride, _lib.stream_ptr(key))
+            _lib.check(rc, "nsa_cache_stage_token")
 
     # ---- after rope ---------------------------------------------------------------------------
     def update_kv(self, cu_seqlens, step, compress_key, compress_value, sparse_key, sparse_value, sliding_key, sliding_value):
         assert compress_key.shape == compress_value.shape and sparse_key.shape == sparse_value.shape
         assert sliding_key.shape == sliding_value.shape
+        batch = cu_seqlens.shape[0] - 1
         if step == 0:
             seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
-            batch = seqlens.shape[0]
-            comp_seqlens, comp_cu = get_compressed_seqlens(cu_seqlens, self.kernel_size, self.kernel_stride)
-            _fill_slab(self.compress_kv_cache, compress_key, compress_value, comp_cu[:-1], comp_cu[1:])
-            self.compress_kv_len[:batch] = comp_seqlens
-            _fill_slab(self.sparse_kv_cache, sparse_key, sparse_value, cu_seqlens[:-1], cu_seqlens[1:])
-            self.sparse_kv_len[:batch] = seqlens
+            self.max_prompt_len = int(seqlens.max())  # the one host read of a prefill
+            assert self.max_prompt_len <= self.max_length
+            _, comp_cu = get_compressed_seqlens(cu_seqlens, self.kernel_size, self.kernel_stride)
+            self._fill(self.compress_kv_cache, self.compress_kv_len, compress_key, compress_value, comp_cu,
+                       comp_cu[:-1].contiguous(), comp_cu[1:].contiguous())
+            self._fill(self.sparse_kv_cache, self.sparse_kv_len, sparse_key, sparse_value, cu_seqlens,
+                       cu_seqlens[:-1].contiguous(), cu_seqlens[1:].contiguous())
             # the last window_size tokens, stored from row 0 (the decode kernel reads the ring as a set)
-            start = torch.maximum(cu_seqlens[1:] - self.window_size, cu_seqlens[:-1])
-            _fill_slab(self.sliding_kv_cache, sliding_key, sliding_value, start, cu_seqlens[1:])
-            self.sliding_kv_len[:batch] = cu_seqlens[1:] - start
+            start = torch.maximum(cu_seqlens[1:] - self.window_size, cu_seqlens[:-1]).contiguous()
+            self._fill(self.sliding_kv_cache, self.sliding_kv_len, sliding_key, sliding_value, cu_seqlens, start, cu_seqlens[1:].contiguous())
         else:
-            batch = sparse_key.shape[0]
-            full = self.before_compress_kv_len[:batch] == self.kernel_size
-            if bool(full.any()):
-                idx = torch.nonzero(full).flatten()
-                at = self.compress_kv_len[idx].long()
-                self.compress_kv_cache[0, idx, at] = compress_key[idx]
-                self.compress_kv_cache[1, idx, at] = compress_value[idx]
-                self.compress_kv_len[idx] += 1
-            rows = torch.arange(batch, device=sparse_key.device)
-            at = self.sparse_kv_len[:batch].long()
-            self.sparse_kv_cache[0, rows, at] = sparse_key
-            self.sparse_kv_cache[1, rows, at] = sparse_value
-            self.sparse_kv_len[:batch] += 1
-            ring = (self.sliding_kv_len[:batch] % self.window_size).long()
-            self.sliding_kv_cache[0, rows, ring] = sliding_key
-            self.sliding_kv_cache[1, rows, ring] = sliding_value
-            self.sliding_kv_len[:batch] += 1
+            assert self.max_seqlen(step) <= self.max_length, "cache slab too short for this decode step"
+            toks = [last_dim_contiguous(t) for t in (compress_key, compress_value, sparse_key, sparse_value, sliding_key, sliding_value)]
+            assert all(t.shape[0] == batch and t.dtype == self.dtype for t in toks)
+            ptrs = (ctypes.c_void_p * 6)(*[t.data_ptr() for t in toks])
+            strides = _lib.host_i64([s for t in toks for s in (t.stride(0), t.stride(1))])
+            rc = _lib.load().nsa_cache_commit_token(
+                ptrs, strides, self.before_compress_kv_len.data_ptr(), self.compress_kv_cache.data_ptr(), self.compress_kv_len.data_ptr(),
+                self.sparse_kv_cache.data_ptr(), self.sparse_kv_len.data_ptr(), self.sliding_kv_cache.data_ptr(),
+                self.sliding_kv_len.data_ptr(), batch, self.num_kv_heads, self.head_dim, self.max_batch_size, self.kernel_size,
+                self.max_comp_length, self.max_length, self.window_size, _lib.stream_ptr(toks[2]))
+            _lib.check(rc, "nsa_cache_commit_token")

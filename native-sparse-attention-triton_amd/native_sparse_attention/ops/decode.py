@@ -77,7 +77,7 @@ def topk_sparse_attention_decode(q, k, v, topk_idx, block_size: int, seqlens, sm
 
 def compressed_attention_decode(
     q, k, v, seqlens, compress_seqlens, kernel_size: int, kernel_stride: int, block_size: int, topk: int,
-    init_blocks: int = 1, local_blocks: int = 2, sm_scale: Optional[float] = None,
+    init_blocks: int = 1, local_blocks: int = 2, sm_scale: Optional[float] = None, max_seqlen: Optional[int] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Attention over the compressed cache plus selection of the blocks for the sparse branch.
 
@@ -85,6 +85,8 @@ def compressed_attention_decode(
     seqlens: uncompressed length of each sequence including the token being decoded; compress_seqlens:
     compressed length.  Returns (out [batch, num_q_heads, head_dim],
     topk_idx int32 [num_kv_heads, batch, min(topk, ceil(max(seqlens) / block_size))]).
+    max_seqlen (not in the reference's signature): max(seqlens) when the caller knows it on the host; the output
+    shape then needs no device read.
     """
     assert block_size % kernel_size == 0 and kernel_size % kernel_stride == 0
     B, Hq, Hkv, D, L = _common_checks(q, k, v, seqlens)
@@ -94,7 +96,8 @@ def compressed_attention_decode(
     if L == 0:  # input too short to have a compressed token
         return torch.zeros_like(q), torch.zeros(Hkv, B, 1, device=q.device, dtype=torch.int32)
     q, k, v = map(last_dim_contiguous, (q, k, v))
-    max_seqlen = int(seqlens.max())  # fixes the output shape; the reference synchronises here too (:30)
+    if max_seqlen is None:
+        max_seqlen = int(seqlens.max())  # fixes the output shape; the reference synchronises here too (:30)
     k_out = min(topk, math.ceil(max_seqlen / block_size))
     o = torch.zeros_like(q, memory_format=torch.contiguous_format)
     idx = torch.empty(Hkv, B, k_out, dtype=torch.int32, device=q.device)

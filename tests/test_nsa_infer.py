@@ -109,3 +109,14 @@ def test_decode_steps_equal_prefill_last_row(device, prompt_lens, steps):
             L = prompt_lens[b] + step
             assert int(cache.sparse_kv_len[b]) == L and int(cache.sliding_kv_len[b]) == min(prompt_lens[b], W) + step
             assert int(cache.compress_kv_len[b]) == (0 if L < ks else (L - ks) // st + 1)
+
+
+@pytest.mark.parametrize("n,H,d,dtype", [(1000, 32, 128, torch.bfloat16), (3, 6, 64, torch.float16), (257, 16, 96, torch.bfloat16)])
+def test_gate_combine_is_bit_identical_to_the_tensor_expression(device, n, H, d, dtype):
+    from native_sparse_attention.infer.nsa_inference import gate_combine
+    g = torch.Generator(device=device).manual_seed(2)
+    gate = torch.sigmoid(torch.randn(n, H * 3, generator=g, device=device)).to(dtype).view(n, H, 3)
+    a, b = (torch.randn(n, H, d, generator=g, device=device).to(dtype) for _ in range(2))
+    c = torch.randn(n, H, 2 * d, generator=g, device=device).to(dtype)[..., :d]   # strided rows
+    want = gate[..., 0, None] * a + gate[..., 1, None] * b + gate[..., 2, None] * c
+    assert torch.equal(gate_combine(gate, a, b, c), want)
