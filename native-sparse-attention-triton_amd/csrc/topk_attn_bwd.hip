@@ -127,7 +127,8 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   __shared__ __attribute__((aligned(16))) T k_s[4][64][LD];
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   typedef short s16x8 __attribute__((ext_vector_type(8)));
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // scalar wave index: token, sequence, block ids and fragment addresses are then computed once per wave
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, lg = lane >> 4;
   const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
   if (item >= p.n_items) return;
@@ -155,8 +156,10 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
 #pragma unroll
   for (int i = 0; i < NDT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
-  const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
-  const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D + lane * 8;
+  const T* kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D;  // wave-uniform; lanes add lane * 8
+  const T* vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D;
+  const unsigned lane8 = lane * 8u;
+  const float dls = dl * p.sm_scale;
   T (*ks)[LD] = k_s[wave];
   const int last_slot = (len - 1) >> 5;
   // block ids are read once (lane e holds entry e) and visited through a wave-uniform bit mask
@@ -181,8 +184,8 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
         const int st = min((key0 >> 4) + nt, 2 * last_slot + 1);  // future sub-tiles: clamp onto existing storage
 #pragma unroll
         for (int kk = 0; kk < NK; kk++) {
-          kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512);
-          vfr[nt][kk] = ld16<v8>(vbase + (long long)(st * NK + kk) * 512);
+          kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512 + lane8);
+          vfr[nt][kk] = ld16<v8>(vbase + (long long)(st * NK + kk) * 512 + lane8);
         }
       }
       f32x4 ds[NS];
@@ -196,11 +199,16 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
           dp = E::mfma16(vfr[nt][kk], dof[kk], dp);
         }
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int key = key0 + 16 * nt + 4 * lg + r;
-          const float pr = key <= pos ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
-          ds[nt][r] = pr * (dp[r] - dl) * p.sm_scale;
-        }
+        for (int r = 0; r < 4; r++)
+          ds[nt][r] = fast_exp2(__builtin_fmaf(s[r], p.qk_scale, -l2)) * __builtin_fmaf(dp[r], p.sm_scale, -dls);
+      }
+      // only the slice that holds the query's own position needs the causal test
+      if (key0 + 16 * NS - 1 > pos) {
+#pragma unroll
+        for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (key0 + 16 * nt + 4 * lg + r > pos) ds[nt][r] = 0.f;
       }
 #pragma unroll
       for (int c = 0; c < (NS + 1) / 2; c++) {
