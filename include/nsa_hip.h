@@ -175,6 +175,24 @@ int nsa_window_attn_bwd(const void* q, const void* k, const void* v, const void*
                         int64_t num_kv_heads, int64_t head_dim, int64_t window_size, const int64_t* strides, float sm_scale,
                         int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- dense varlen attention ------------------------------------------------------------------
+ * Replaces _flash_attention_fwd / _flash_attention_bwd behind flash_attention_varlen
+ * (native_sparse_attention/ops/triton/flash_attention.py:560-935): q [total_q, Hq, D], k/v [total_k, Hkv, D],
+ * separate cu_seqlens for queries and keys; causal != 0: query i of a sequence sees keys j <= i of the same
+ * sequence (both counted from their start, :117-131), otherwise every key.  lse fp32 [Hq, total_q], base 2.
+ * Strides as for the sliding-window entry points (HOST int64[8] forward, int64[16] backward).
+ */
+int nsa_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens_q,
+                       const int32_t* cu_seqlens_k, int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads,
+                       int64_t num_kv_heads, int64_t head_dim, int causal, const int64_t* strides, float sm_scale, int dtype,
+                       void* stream);
+size_t nsa_flash_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                          int64_t head_dim);
+int nsa_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse, void* dq, void* dk,
+                       void* dv, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q, int64_t total_k,
+                       int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int causal, const int64_t* strides,
+                       float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- rotary position embedding ---------------------------------------------------------------
  * Replaces RotaryEmbedding.forward of native_sparse_attention/module/rope.py:199-209 (cos/sin tables
  * :120-152, per-sequence positions :154-197): x, out [n_rows, H, D] (strides in elements, multiples of 8),

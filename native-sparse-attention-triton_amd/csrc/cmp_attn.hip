@@ -21,7 +21,7 @@ struct CmpParams {
   const void* q; const void* k; const void* v; const void* dout; void* o; void* dq; float* lse; const float* delta;
   const int32_t* cu_q; const int32_t* cu_k;
   int total_q, batch, Hkv, G, GT, ks, st;
-  int window;  // < 0: compressed keys (rule above); >= 0: ordinary keys, position i sees j in [i - window, i]
+  int window;  // -1: compressed keys (rule above); >= 0: ordinary keys, position i sees j in [i - window, i]; -2: ordinary keys, all visible
   long long qsn, qsh, ksn, ksh, vsn, vsh, osn, osh, dsn, dsh, dqsn, dqsh;
   float qk_scale, sm_scale;
 };
@@ -51,7 +51,10 @@ __device__ __forceinline__ int visible_keys(int pos, int lq, int lk, int ks, int
 
 // half-open range [lo, hi) of keys visible to position pos
 __device__ __forceinline__ void visible_range(int pos, int lq, int lk, int ks, int st, int window, int& lo, int& hi) {
-  if (window < 0) {
+  if (window == -2) {
+    lo = 0;
+    hi = pos < lq ? lk : 0;
+  } else if (window < 0) {
     lo = 0;
     hi = visible_keys(pos, lq, lk, ks, st);
   } else {
@@ -640,10 +643,10 @@ __global__ void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int3
     for (int b = 0; b < batch; b++) {
       const int lq = cu_q[b + 1] - cu_q[b];
       for (int g = cu_blk[b]; g < cu_blk[b + 1]; g++) {
-        const int first_pos = (g - cu_blk[b]) * 64 * st + ks - 1;
+        const int first_pos = window == -2 ? 0 : (g - cu_blk[b]) * 64 * st + ks - 1;
         seg_begin[h * max_blocks + g] = cu_q[b] + min(first_pos, lq);
         // window mode (ordinary keys): the block's last key 64*g' + 63 is seen up to position 64*g' + 63 + window
-        seg_end[h * max_blocks + g] = cu_q[b] + (window < 0 ? lq : (int)min((long long)lq, (long long)(g - cu_blk[b]) * 64 + 64 + window));
+        seg_end[h * max_blocks + g] = cu_q[b] + (window < 0 ? lq : (int)min((long long)lq, (long long)(g - cu_blk[b]) * 64 + 64 + window));  // -1, -2: to the end
       }
     }
   }
@@ -849,6 +852,48 @@ extern "C" int nsa_window_attn_bwd(const void* q, const void* k, const void* v, 
   a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
   a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
   a.p.window = (int)(window_size > (1 << 30) ? (1 << 30) : window_size);
+  a.ws = (char*)workspace;
+  a.what = 2;
+  return cmp_dispatch(a, head_dim, dtype);
+}
+
+// Dense varlen attention with separate query / key lengths per sequence (causal: query i sees keys j <= i, counted
+// from the start of both; otherwise every key): the same tile kernels once more.
+extern "C" size_t nsa_flash_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
+                                                     int64_t head_dim) {
+  return cmp_bwd_layout(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim).total;
+}
+
+extern "C" int nsa_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens_q,
+                                  const int32_t* cu_seqlens_k, int64_t total_q, int64_t total_k, int64_t batch, int64_t num_q_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int causal, const int64_t* strides, float sm_scale, int dtype,
+                                  void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, v, cu_seqlens_q, cu_seqlens_k, total_q, total_k, batch, num_q_heads, num_kv_heads, 1, 1, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!v || !o || !lse || strides[6] % 4 != 0 || strides[7] % 4 != 0 || (uintptr_t)o % 8 != 0) return NSA_ERR_BAD_ARG;
+  a.p.o = o; a.p.lse = lse; a.p.osn = strides[6]; a.p.osh = strides[7];
+  a.p.window = causal ? (1 << 30) : -2;
+  a.what = 0;
+  return cmp_dispatch(a, head_dim, dtype);
+}
+
+extern "C" int nsa_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse, void* dq,
+                                  void* dk, void* dv, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q,
+                                  int64_t total_k, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int causal,
+                                  const int64_t* strides, float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  CmpArgs a;
+  int rc = cmp_common(a, q, k, v, cu_seqlens_q, cu_seqlens_k, total_q, total_k, batch, num_q_heads, num_kv_heads, 1, 1, strides, sm_scale, dtype, stream);
+  if (rc != NSA_OK) return rc;
+  if (!v || !o || !dout || !lse || !dq || !dk || !dv || !workspace) return NSA_ERR_BAD_ARG;
+  for (int i = 6; i < 10; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
+  for (int i = 10; i < 16; i++) if (strides[i] % 4 != 0) return NSA_ERR_UNSUPPORTED;
+  if (((uintptr_t)o | (uintptr_t)dout) % 16 != 0 || ((uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) % 8 != 0 || (uintptr_t)workspace % 256 != 0) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_flash_attn_bwd_workspace_bytes(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
+  a.o_in = o; a.p.dout = dout; a.p.lse = (float*)lse; a.p.dq = dq; a.dk = dk; a.dv = dv;
+  a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
+  a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
+  a.p.window = causal ? (1 << 30) : -2;
   a.ws = (char*)workspace;
   a.what = 2;
   return cmp_dispatch(a, head_dim, dtype);

@@ -50,7 +50,7 @@ struct DkdvParams {
   const int32_t* cu; const int32_t* cu_k; const int32_t* cu_blk; const int32_t* seg_begin; const int32_t* seg_end; const int32_t* chunk_off; const int32_t* queries;
   float* partial;
   int total_len, batch, Hkv, G, GT, max_blocks, n_seg, ks, st;
-  int window;  // range mode: < 0 compressed keys (key c seen from position c*st + ks - 1 on), >= 0 ordinary keys seen by [key, key + window]
+  int window;  // range mode: -1 compressed keys (key c seen from position c*st + ks - 1 on), >= 0 ordinary keys seen by [key, key + window], -2 every key seen by every position
   long long ksn, ksh, vsn, vsh;
   int qsn, qsh, dsn, dsh;  // element strides of q / dO (checked on the host to fit 31 bits)
   float qk_scale, sm_scale;
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
         for (int r = 0; r < 4; r++) {
           const float l2 = l4[r];
           const float dl = d4[r];
-          const bool vis = RANGE ? (key < len && key * p.st + p.ks - 1 <= pos && (p.window < 0 || key >= pos - p.window)) : key <= pos;
+          const bool vis = RANGE ? (key < len && (p.window == -2 || (key * p.st + p.ks - 1 <= pos && (p.window < 0 || key >= pos - p.window)))) : key <= pos;
           const float pr = fast_exp2(vis ? s[r] * p.qk_scale - l2 : -INFINITY);  // select, not a branch
           pf[j][tk * 4 + r] = (T)pr;
           dsf[j][tk * 4 + r] = (T)(pr * (dp[r] - dl) * p.sm_scale);
