@@ -12,11 +12,14 @@ import torch
 
 from .. import _lib
 from ..ops import (
+    avgpool_compress,
     compressed_attention,
     compressed_attention_decode,
     flash_attention_decode,
+    linear_compress,
     topk_sparse_attention,
     topk_sparse_attention_decode,
+    weightedpool_compress,
 )
 from ..ops.sliding_window import sliding_window_attention_varlen
 from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
@@ -29,13 +32,21 @@ def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, i
         return key, value, compress_cu_seqlens
     # decode: compress every sequence's staging window -> exactly one candidate token per sequence
     batch = cu_seqlens.shape[0] - 1
-    aux_cu = torch.arange(batch + 1, dtype=torch.int32, device=cu_seqlens.device) * kernel_size
+    aux_cu = cache.staging_cu_seqlens(batch)
     stage = cache.before_compress_kv_cache[:, :batch].reshape(2, batch * kernel_size, cache.num_kv_heads, cache.head_dim)
-    key, _ = compress_func[0](stage[0], weight[0], aux_cu, kernel_size, kernel_stride, intra_block_pe)
-    value, _ = compress_func[1](stage[1], weight[1], aux_cu, kernel_size, kernel_stride)
+    key, _ = _compress_known_total(compress_func[0], batch, stage[0], weight[0], aux_cu, kernel_size, kernel_stride, intra_block_pe)
+    value, _ = _compress_known_total(compress_func[1], batch, stage[1], weight[1], aux_cu, kernel_size, kernel_stride)
     compress_cu_seqlens = torch.zeros(batch + 1, dtype=torch.int32, device=key.device)
     compress_cu_seqlens[1:] = torch.cumsum(cache.compress_kv_len[:batch], dim=0)  # lengths before this token
     return key, value, compress_cu_seqlens
+
+
+def _compress_known_total(func, total, *args):
+    """Call a compression operator; this package's own operators are told the (host-known) number of output rows so
+    that they need not read it back from the device, any other callable gets the reference's arguments only."""
+    if func in (weightedpool_compress, avgpool_compress, linear_compress):
+        return func(*args, known_total=total)
+    return func(*args)
 
 
 def compressed_attention_infer(cu_seqlens, step, query, key, value, cache, kernel_size, kernel_stride, topk, block_size,

@@ -36,6 +36,7 @@ class NSACache:
         self.dtype, self.device = dtype, device
         self.max_comp_length = (max_length - kernel_size) // kernel_stride + 1
         self.max_prompt_len = 0  # host copy of the longest prompt of the current batch (set at prefill)
+        self._staging_cu = None
 
         def slab(rows):
             return torch.zeros(2, max_batch_size, rows, num_kv_heads, head_dim, dtype=dtype, device=device)
@@ -53,6 +54,12 @@ class NSACache:
         for t in (self.sparse_kv_len, self.compress_kv_len, self.before_compress_kv_len, self.sliding_kv_len):
             t.zero_()
         self.max_prompt_len = 0
+
+    def staging_cu_seqlens(self, batch: int) -> torch.Tensor:
+        """cu_seqlens of the staging slab seen as a varlen batch: every sequence contributes kernel_size rows."""
+        if self._staging_cu is None:
+            self._staging_cu = torch.arange(self.max_batch_size + 1, dtype=torch.int32, device=self.device) * self.kernel_size
+        return self._staging_cu[: batch + 1]
 
     def max_seqlen(self, step: int) -> int:
         """Upper bound, known on the host, of every sequence's length at decode step `step`."""

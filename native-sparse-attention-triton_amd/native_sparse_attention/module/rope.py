@@ -102,10 +102,23 @@ class RotaryEmbedding(nn.Module):
         self.config = config
         inv_freq, self.attention_scaling = compute_inv_freq(config, device)
         self.register_buffer("inv_freq", inv_freq.contiguous(), persistent=False)
+        self._inv_freq_f32 = None
+
+    def _frequencies(self):
+        """fp32 view of the buffer for the kernel.  Casting the module (`.bfloat16()`, `.half()`) casts the buffer
+        too, as it does in the reference, whose forward then widens the rounded values again (rope.py:127-129):
+        the same rounded frequencies are used here."""
+        f = self.inv_freq
+        if f.dtype == torch.float32 and f.is_contiguous():
+            return f
+        c = self._inv_freq_f32
+        if c is None or c[0] is not f:
+            self._inv_freq_f32 = c = (f, f.float().contiguous())
+        return c[1]
 
     def forward(self, x, cu_seqlens, step=0, stride=1):
         assert x.dim() == 3 and x.shape[-1] == self.config.head_dim
         assert x.dtype == torch.bfloat16 or x.dtype == torch.float16
         cu_seqlens = cu_seqlens.to(torch.int32)
         assert step >= 0 and (step == 0 or x.shape[0] == cu_seqlens.shape[0] - 1)
-        return _Rope.apply(x, self.inv_freq, float(self.attention_scaling), cu_seqlens, int(step), int(stride))
+        return _Rope.apply(x, self._frequencies(), float(self.attention_scaling), cu_seqlens, int(step), int(stride))

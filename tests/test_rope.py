@@ -93,3 +93,20 @@ def test_decode_positions(device):
         y = rope(x, cu, step=step, stride=stride)
         want = _reference_forward(x, rope.inv_freq, pos)
         assert ((y.float() - want.float()).abs() <= 2.0 ** -7 * want.float().abs().clamp(min=1.0)).all()
+
+
+@pytest.mark.gpu
+def test_module_cast_to_bf16_rounds_the_frequencies_like_the_reference(device):
+    """`.bfloat16()` on the owning module casts the inv_freq buffer (in the reference too, whose forward widens the
+    rounded values again): the kernel must be handed fp32 copies of those rounded values, not the 2-byte buffer."""
+    lens, H, d = [50, 20], 2, 64
+    cu = cu_from_lens(lens, device)
+    rope = RotaryEmbedding(RopeConfig(head_dim=d), device=device).bfloat16()
+    assert rope.inv_freq.dtype == torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(3)
+    x = torch.randn(sum(lens), H, d, generator=g, device=device).bfloat16()
+    pos = torch.cat([torch.arange(L, device=device) for L in lens])
+    y = rope(x, cu)
+    want = _reference_forward(x, rope.inv_freq.float(), pos)
+    assert torch.isfinite(y).all()
+    assert ((y.float() - want.float()).abs() <= 2.0 ** -7 * want.float().abs().clamp(min=1.0)).all()
