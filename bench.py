@@ -193,7 +193,8 @@ def bench_decode(args, dev):
     gate = torch.sigmoid(torch.randn(T, Hq, 3, generator=g, device=dev)).bfloat16()
     wk = torch.softmax(torch.randn(Hkv, ks, generator=g, device=dev), -1).bfloat16()
     wv = torch.softmax(torch.randn(Hkv, ks, generator=g, device=dev), -1).bfloat16()
-    rope = lambda x, c, s, stride=1: x
+    from native_sparse_attention.module import RopeConfig, RotaryEmbedding
+    rope = RotaryEmbedding(RopeConfig(head_dim=D), device=dev)  # llama3 rotary embedding, as the layer applies it
     steps = max(4, args.steps)
     cache = NSACache(B, max(lens) + steps + 8, Hkv, D, ks, st, W, torch.bfloat16, dev)
     fargs = (rope, cache, (wk, wv), (weightedpool_compress, weightedpool_compress), None, ks, st, bs, topk, 1, 2, W)

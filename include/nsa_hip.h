@@ -193,13 +193,23 @@ int nsa_flash_attn_bwd(const void* q, const void* k, const void* v, const void* 
                        int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int causal, const int64_t* strides,
                        float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- compressed sequence lengths ---------------------------------------------------------------
+ * get_compressed_seqlens of native_sparse_attention/ops/triton/utils.py:25-37 in one launch:
+ * y_seqlens[b] = floor((len_b - kernel_size) / kernel_stride) + 1, or 0 when len_b < kernel_size; y_cu_seqlens =
+ * its cumulative sum with a leading 0 (int32 [batch] and [batch + 1], device).
+ */
+int nsa_compressed_seqlens(const int32_t* cu_seqlens, int64_t batch, int64_t kernel_size, int64_t kernel_stride,
+                           int32_t* y_seqlens, int32_t* y_cu_seqlens, void* stream);
+
 /* ---- rotary position embedding ---------------------------------------------------------------
  * Replaces RotaryEmbedding.forward of native_sparse_attention/module/rope.py:199-209 (cos/sin tables
  * :120-152, per-sequence positions :154-197): x, out [n_rows, H, D] (strides in elements, multiples of 8),
  * inv_freq fp32 [D/2] on the device.  step == 0: row n is token (n - cu_seqlens[b]) of sequence b and is
  * rotated for position (n - cu_seqlens[b]) * stride.  step > 0 (decode): n_rows == batch, row b is rotated
- * for position (cu_seqlens[b+1] - cu_seqlens[b] + step - 1) * stride.  inverse != 0 applies the transposed
- * rotation (the gradient of the forward call).
+ * for position (cu_seqlens[b+1] - cu_seqlens[b] + step - 1) * stride.  step < 0: cu_seqlens is instead an
+ * int32 [n_rows] array of position indices on the device (row n is rotated for position index * stride; batch is
+ * ignored), which lets a decode step take positions from the cache lengths without a host read.  inverse != 0
+ * applies the transposed rotation (the gradient of the forward call).
  */
 int nsa_rope(const void* x, void* out, const float* inv_freq, const int32_t* cu_seqlens, int64_t n_rows, int64_t batch,
              int64_t num_heads, int64_t head_dim, int64_t x_stride_n, int64_t x_stride_h, int64_t o_stride_n, int64_t o_stride_h,

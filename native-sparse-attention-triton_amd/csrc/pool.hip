@@ -197,3 +197,42 @@ extern "C" int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* 
   POOL_DISPATCH(CALL)
 #undef CALL
 }
+
+// y_len[b] = floor((len_b - ks) / st) + 1 (0 when len_b < ks) and its cumulative sum, in one launch
+// (native_sparse_attention/ops/triton/utils.py:25-37 of the reference spends a dozen tensor-op launches on it).
+__global__ __launch_bounds__(256) void compressed_seqlens_kernel(const int32_t* __restrict__ cu, int batch, int ks, int st,
+                                                                 int32_t* __restrict__ y_len, int32_t* __restrict__ y_cu) {
+  __shared__ int part[256];
+  const int tid = threadIdx.x;
+  // thread t owns sequences [t*per, (t+1)*per)
+  const int per = (batch + 255) / 256;
+  int sum = 0;
+  for (int b = tid * per; b < min(batch, (tid + 1) * per); b++) {
+    const int len = cu[b + 1] - cu[b];
+    const int n = len < ks ? 0 : (len - ks) / st + 1;
+    y_len[b] = n;
+    sum += n;
+  }
+  part[tid] = sum;
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {
+    const int v = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - sum;  // exclusive prefix of this thread's sequences
+  if (tid == 0) y_cu[0] = 0;
+  for (int b = tid * per; b < min(batch, (tid + 1) * per); b++) {
+    const int len = cu[b + 1] - cu[b];
+    run += len < ks ? 0 : (len - ks) / st + 1;
+    y_cu[b + 1] = run;
+  }
+}
+
+extern "C" int nsa_compressed_seqlens(const int32_t* cu_seqlens, int64_t batch, int64_t kernel_size, int64_t kernel_stride,
+                                      int32_t* y_seqlens, int32_t* y_cu_seqlens, void* stream) {
+  if (!cu_seqlens || !y_seqlens || !y_cu_seqlens || batch <= 0 || kernel_size <= 0 || kernel_stride <= 0 || batch >= (1ll << 31)) return NSA_ERR_BAD_ARG;
+  compressed_seqlens_kernel<<<1, 256, 0, (hipStream_t)stream>>>(cu_seqlens, (int)batch, (int)kernel_size, (int)kernel_stride, y_seqlens, y_cu_seqlens);
+  return nsa_check_launch();
+}

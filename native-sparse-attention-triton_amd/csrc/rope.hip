@@ -22,7 +22,9 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
   __shared__ float cos_s[HALF], sin_s[HALF];
   const int n = blockIdx.x;
   int pos;
-  if (p.step == 0) {  // prefill: row n is token n - cu[b] of its sequence
+  if (p.step < 0) {   // the caller supplies one position index per row
+    pos = p.cu[n] * p.stride;
+  } else if (p.step == 0) {  // prefill: row n is token n - cu[b] of its sequence
     const int b = find_sequence(p.cu, p.batch, n);
     pos = (n - p.cu[b]) * p.stride;
   } else {            // decode: one row per sequence, `step` tokens after its prompt
@@ -70,7 +72,7 @@ extern "C" int nsa_rope(const void* x, void* out, const float* inv_freq, const i
                         int64_t o_stride_h, int64_t step, int64_t stride, float attention_scaling, int inverse, int dtype,
                         void* stream) {
   if (!x || !out || !inv_freq || !cu_seqlens) return NSA_ERR_BAD_ARG;
-  if (n_rows < 0 || batch <= 0 || num_heads <= 0 || step < 0 || stride <= 0 || n_rows >= (1ll << 31)) return NSA_ERR_BAD_ARG;
+  if (n_rows < 0 || batch <= 0 || num_heads <= 0 || stride <= 0 || n_rows >= (1ll << 31)) return NSA_ERR_BAD_ARG;
   if (step > 0 && n_rows != batch) return NSA_ERR_BAD_ARG;
   if ((x_stride_n | x_stride_h | o_stride_n | o_stride_h) % 8 != 0 || ((uintptr_t)x | (uintptr_t)out) % 16 != 0) return NSA_ERR_UNSUPPORTED;
   if (n_rows == 0) return NSA_OK;

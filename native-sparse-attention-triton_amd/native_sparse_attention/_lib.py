@@ -46,6 +46,7 @@ _SIGNATURES = {
     "nsa_flash_attn_fwd": (c_int, [P] * 7 + [I] * 6 + [c_int, P, F, c_int, P]),
     "nsa_flash_attn_bwd_workspace_bytes": (Z, [I] * 6),
     "nsa_flash_attn_bwd": (c_int, [P] * 11 + [I] * 6 + [c_int, P, F, c_int, P, Z, P]),
+    "nsa_compressed_seqlens": (c_int, [P] + [I] * 3 + [P, P, P]),
     "nsa_rope": (c_int, [P] * 4 + [I] * 10 + [F, c_int, c_int, P]),
     "nsa_window_attn_bwd_workspace_bytes": (Z, [I] * 5),
     "nsa_window_attn_bwd": (c_int, [P] * 10 + [I] * 6 + [P, F, c_int, P, Z, P]),

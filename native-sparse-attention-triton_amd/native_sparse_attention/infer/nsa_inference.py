@@ -25,7 +25,8 @@ from ..ops.sliding_window import sliding_window_attention_varlen
 from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
 
 
-def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, intra_block_pe, kernel_size, kernel_stride):
+def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, intra_block_pe, kernel_size, kernel_stride,
+                   need_cu=True):
     if step == 0:
         key, compress_cu_seqlens = compress_func[0](key, weight[0], cu_seqlens, kernel_size, kernel_stride, intra_block_pe)
         value, _ = compress_func[1](value, weight[1], cu_seqlens, kernel_size, kernel_stride)
@@ -36,6 +37,8 @@ def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, i
     stage = cache.before_compress_kv_cache[:, :batch].reshape(2, batch * kernel_size, cache.num_kv_heads, cache.head_dim)
     key, _ = _compress_known_total(compress_func[0], batch, stage[0], weight[0], aux_cu, kernel_size, kernel_stride, intra_block_pe)
     value, _ = _compress_known_total(compress_func[1], batch, stage[1], weight[1], aux_cu, kernel_size, kernel_stride)
+    if not need_cu:
+        return key, value, None
     compress_cu_seqlens = torch.zeros(batch + 1, dtype=torch.int32, device=key.device)
     compress_cu_seqlens[1:] = torch.cumsum(cache.compress_kv_len[:batch], dim=0)  # lengths before this token
     return key, value, compress_cu_seqlens
@@ -57,7 +60,7 @@ def compressed_attention_infer(cu_seqlens, step, query, key, value, cache, kerne
         return compressed_attention(query, key, value, kernel_size, kernel_stride, block_size, topk, cu_seqlens, comp_cu,
                                     int(seqlens.max()), int(comp_seqlens.max()), None, init_blocks, local_blocks)
     batch = cu_seqlens.shape[0] - 1
-    seqlens = cu_seqlens[1:] - cu_seqlens[:-1] + step
+    seqlens = cache.sparse_kv_len[:batch]  # prompt length + step once the new token is in the cache
     # slab rows that can hold a compressed token at this step, from the host-side length bound (the reference
     # slices by compress_kv_len.max(), inference_func.py:127-135, which waits for the device)
     max_seqlen = cache.max_seqlen(step)
@@ -79,8 +82,9 @@ def sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, w
     if step == 0:
         return sliding_window_attention_varlen(query, key, value, cu_seqlens, window_size)
     batch = cu_seqlens.shape[0] - 1
-    lens = torch.clamp(cache.sliding_kv_len[:batch], max=window_size)
-    return flash_attention_decode(query, cache.sliding_kv_cache[0, :batch], cache.sliding_kv_cache[1, :batch], lens)
+    # the ring holds min(tokens seen, window_size) rows; the kernel clips the count to the slab by itself
+    return flash_attention_decode(query, cache.sliding_kv_cache[0, :batch], cache.sliding_kv_cache[1, :batch],
+                                  cache.sliding_kv_len[:batch])
 
 
 def gate_combine(gate_value, branch0, branch1, branch2):
@@ -123,11 +127,21 @@ def nsa_infer(
     if step == 0:
         cache.reset()
     cache.prepare_compress(cu_seqlens, step, key, value)
+    # In a decode step every position is a cache length that lives on the device: this package's rotary module can
+    # take them from there, any other rope callable gets the reference's (cu_seqlens, step) arguments.
+    on_device_positions = step > 0 and hasattr(rope, "rotate_at")
     compress_key, compress_value, compress_cu = compress_infer(
-        cu_seqlens, step, key, value, cache, compress_weight, compress_func, intra_block_pe, kernel_size, kernel_stride)
-    query = rope(query, cu_seqlens, step)
-    compress_key = rope(compress_key, compress_cu, step if step == 0 else 1, stride=cache.kernel_stride)
-    key = rope(key, cu_seqlens, step)
+        cu_seqlens, step, key, value, cache, compress_weight, compress_func, intra_block_pe, kernel_size, kernel_stride,
+        need_cu=not on_device_positions)
+    if on_device_positions:
+        batch = cu_seqlens.shape[0] - 1
+        query = rope.rotate_at(query, cache.sparse_kv_len[:batch])
+        key = rope.rotate_at(key, cache.sparse_kv_len[:batch])
+        compress_key = rope.rotate_at(compress_key, cache.compress_kv_len[:batch], stride=cache.kernel_stride)
+    else:
+        query = rope(query, cu_seqlens, step)
+        compress_key = rope(compress_key, compress_cu, step if step == 0 else 1, stride=cache.kernel_stride)
+        key = rope(key, cu_seqlens, step)
     cache.update_kv(cu_seqlens, step, compress_key, compress_value, key, value, key, value)
     cmp_out, topk_idx = compressed_attention_infer(cu_seqlens, step, query, compress_key, compress_value, cache, kernel_size,
                                                    kernel_stride, topk, block_size, init_blocks, local_blocks)

@@ -68,7 +68,7 @@ def compute_inv_freq(config: RopeConfig, device=None):
 def _rope_launch(x, inv_freq, scaling, cu_seqlens, step, stride, inverse):
     x = last_dim_contiguous(x)
     out = torch.empty_like(x, memory_format=torch.contiguous_format)
-    B = cu_seqlens.shape[0] - 1
+    B = max(cu_seqlens.shape[0] - 1, 1)  # ignored when cu_seqlens carries positions (step < 0)
     rc = _lib.load().nsa_rope(x.data_ptr(), out.data_ptr(), inv_freq.data_ptr(), cu_seqlens.data_ptr(), x.shape[0], B, x.shape[1],
                               x.shape[2], x.stride(0), x.stride(1), out.stride(0), out.stride(1), step, stride, scaling,
                               int(inverse), _lib.dtype_code(x), _lib.stream_ptr(x))
@@ -115,6 +115,14 @@ class RotaryEmbedding(nn.Module):
         if c is None or c[0] is not f:
             self._inv_freq_f32 = c = (f, f.float().contiguous())
         return c[1]
+
+    @torch.no_grad()
+    def rotate_at(self, x, position_index, stride=1):
+        """Rotate row n of x [N, H, D] for position position_index[n] * stride, position_index an int32 tensor [N] on the
+        device (e.g. the cache's length vector): no host knowledge of the positions is needed.  No autograd."""
+        assert x.dim() == 3 and x.shape[-1] == self.config.head_dim and position_index.dtype == torch.int32
+        assert position_index.shape[0] == x.shape[0] and position_index.is_contiguous()
+        return _rope_launch(x, self._frequencies(), float(self.attention_scaling), position_index, -1, int(stride), False)
 
     def forward(self, x, cu_seqlens, step=0, stride=1):
         assert x.dim() == 3 and x.shape[-1] == self.config.head_dim

@@ -9,6 +9,15 @@ def get_compressed_seqlens(cu_seqlens: torch.Tensor, kernel_size: int, kernel_st
     int32 on the device of ``cu_seqlens`` (same contract as the reference's
     native_sparse_attention/ops/triton/utils.py:25-37).
     """
+    if cu_seqlens.is_cuda and cu_seqlens.dtype == torch.int32 and cu_seqlens.is_contiguous():
+        from .. import _lib  # one launch instead of a dozen tensor operations
+        batch = cu_seqlens.shape[0] - 1
+        y_seqlens = torch.empty(batch, dtype=torch.int32, device=cu_seqlens.device)
+        y_cu_seqlens = torch.empty(batch + 1, dtype=torch.int32, device=cu_seqlens.device)
+        rc = _lib.load().nsa_compressed_seqlens(cu_seqlens.data_ptr(), batch, kernel_size, kernel_stride, y_seqlens.data_ptr(),
+                                                y_cu_seqlens.data_ptr(), _lib.stream_ptr(cu_seqlens))
+        _lib.check(rc, "nsa_compressed_seqlens")
+        return y_seqlens, y_cu_seqlens
     seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
     y_seqlens = torch.div(seqlens - kernel_size, kernel_stride, rounding_mode="floor").to(torch.int32) + 1
     y_seqlens = torch.where(seqlens < kernel_size, torch.zeros_like(y_seqlens), y_seqlens)
