@@ -63,7 +63,9 @@ def compressed_attention_infer(cu_seqlens, step, query, key, value, cache, kerne
     seqlens = cache.sparse_kv_len[:batch]  # prompt length + step once the new token is in the cache
     # slab rows that can hold a compressed token at this step, from the host-side length bound (the reference
     # slices by compress_kv_len.max(), inference_func.py:127-135, which waits for the device)
-    max_seqlen = cache.max_seqlen(step)
+    # (a cache marked static_shapes always passes its full extents, so that a captured step stays valid as sequences grow:
+    # the kernels bound their work by the per-sequence lengths anyway; ids of blocks a sequence has not reached come out as -1)
+    max_seqlen = cache.max_length if cache.static_shapes else cache.max_seqlen(step)
     rows = min(max((max_seqlen - kernel_size) // kernel_stride + 1, 0), cache.max_comp_length)
     return compressed_attention_decode(query, cache.compress_kv_cache[0, :batch, :rows], cache.compress_kv_cache[1, :batch, :rows],
                                        seqlens, cache.compress_kv_len[:batch], kernel_size, kernel_stride, block_size, topk,

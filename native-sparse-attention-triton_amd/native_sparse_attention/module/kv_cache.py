@@ -37,6 +37,7 @@ class NSACache:
         self.max_comp_length = (max_length - kernel_size) // kernel_stride + 1
         self.max_prompt_len = 0  # host copy of the longest prompt of the current batch (set at prefill)
         self._staging_cu = None
+        self.static_shapes = False  # decode steps use the full slab extents instead of the current length bound
 
         def slab(rows):
             return torch.zeros(2, max_batch_size, rows, num_kv_heads, head_dim, dtype=dtype, device=device)
@@ -112,7 +113,7 @@ class NSACache:
             start = torch.maximum(cu_seqlens[1:] - self.window_size, cu_seqlens[:-1]).contiguous()
             self._fill(self.sliding_kv_cache, self.sliding_kv_len, sliding_key, sliding_value, cu_seqlens, start, cu_seqlens[1:].contiguous())
         else:
-            assert self.max_seqlen(step) <= self.max_length, "cache slab too short for this decode step"
+            assert self.static_shapes or self.max_seqlen(step) <= self.max_length, "cache slab too short for this decode step"
             toks = [last_dim_contiguous(t) for t in (compress_key, compress_value, sparse_key, sparse_value, sliding_key, sliding_value)]
             assert all(t.shape[0] == batch and t.dtype == self.dtype for t in toks)
             ptrs = (ctypes.c_void_p * 6)(*[t.data_ptr() for t in toks])

@@ -120,3 +120,39 @@ def test_gate_combine_is_bit_identical_to_the_tensor_expression(device, n, H, d,
     c = torch.randn(n, H, 2 * d, generator=g, device=device).to(dtype)[..., :d]   # strided rows
     want = gate[..., 0, None] * a + gate[..., 1, None] * b + gate[..., 2, None] * c
     assert torch.equal(gate_combine(gate, a, b, c), want)
+
+
+def test_graphed_decode_step_equals_eager_steps(device):
+    """The decode step recorded in a HIP graph, replayed for many tokens with eager work in between, against the eager
+    decode steps on an identically prefilled second cache."""
+    from native_sparse_attention.infer import NSADecodeGraph
+    from native_sparse_attention.module import RopeConfig, RotaryEmbedding
+    Hq, Hkv, d, ks, st, bs, topk, W = 32, 2, 128, 32, 16, 64, 8, 128
+    lens, steps = [300, 47, 1100], 40
+    B = len(lens)
+    g = torch.Generator(device=device).manual_seed(5)
+    cu = cu_from_lens(lens, device)
+    T = int(cu[-1])
+    rope = RotaryEmbedding(RopeConfig(head_dim=d), device=device)
+    wk = torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).bfloat16()
+    wv = torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).bfloat16()
+    pe = (torch.randn(Hkv, ks, d, generator=g, device=device) * 0.02).bfloat16()
+
+    def rnd(*shape):
+        return torch.randn(*shape, generator=g, device=device).bfloat16()
+
+    q0, k0, v0, g0 = rnd(T, Hq, d), rnd(T, Hkv, d), rnd(T, Hkv, d), torch.sigmoid(rnd(T, Hq, 3).float()).bfloat16()
+    caches = [NSACache(B, max(lens) + steps + 8, Hkv, d, ks, st, W, torch.bfloat16, device) for _ in range(2)]
+    tail = ((wk, wv), (weightedpool_compress, weightedpool_compress), pe, ks, st, bs, topk, 1, 2, W)
+    outs = [nsa_infer(cu, 0, q0, k0, v0, g0, rope, c, *tail) for c in caches]
+    assert torch.equal(outs[0], outs[1])
+    graph = NSADecodeGraph(cu, Hq, rope, caches[0], *tail)
+    for step in range(1, steps + 1):
+        q, k, v, gt = rnd(B, Hq, d), rnd(B, Hkv, d), rnd(B, Hkv, d), torch.sigmoid(rnd(B, Hq, 3).float()).bfloat16()
+        want = nsa_infer(cu, step, q, k, v, gt, rope, caches[1], *tail)
+        got = graph.step(q, k, v, gt)
+        assert_close(got, want.float(), "graph replay %d" % step)
+        for name in ("sparse_kv_len", "compress_kv_len", "before_compress_kv_len", "sliding_kv_len"):
+            assert torch.equal(getattr(caches[0], name), getattr(caches[1], name)), (name, step)
+    n = int(caches[1].sparse_kv_len[2])
+    assert torch.equal(caches[0].sparse_kv_cache[:, 2, :n], caches[1].sparse_kv_cache[:, 2, :n])
