@@ -131,28 +131,54 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
   }
 }
 
-// merge the chunk partials of one (sequence, query head); optionally keep the base-2 LSE
+// merge the chunk partials of one (sequence, query head); optionally keep the base-2 LSE.  The chunk maxima and
+// sums are read by different threads (independent loads, not a serial chain), the per-chunk weights go through LDS.
 template <typename T, int D>
 __global__ void decode_merge_kernel(DecodeParams p, T* __restrict__ o, long long osb, long long osh, float* __restrict__ lse) {
-  const int hq_all = blockIdx.x, b = blockIdx.y;
+  constexpr int WCAP = 256;  // chunk weights kept in LDS at a time
+  __shared__ float red[128];
+  __shared__ float w_s[WCAP];
+  const int hq_all = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
   const int h = hq_all / p.G, hq = hq_all % p.G, gt = hq / 16, col = hq % 16;
   const long long base = (((long long)b * p.Hkv + h) * p.GT + gt) * p.n_chunks;
   float m = -INFINITY;
-  for (int c = 0; c < p.n_chunks; c++) m = fmaxf(m, p.pm[(base + c) * 16 + col]);
+  for (int c = tid; c < p.n_chunks; c += nt) m = fmaxf(m, p.pm[(base + c) * 16 + col]);
+  red[tid] = m;
+  __syncthreads();
+  for (int s = nt / 2; s > 0; s >>= 1) {
+    if (tid < s) red[tid] = fmaxf(red[tid], red[tid + s]);
+    __syncthreads();
+  }
+  m = red[0];
+  __syncthreads();
   float l = 0.f;
-  for (int c = 0; c < p.n_chunks; c++) {
+  for (int c = tid; c < p.n_chunks; c += nt) {
     const float mc = p.pm[(base + c) * 16 + col];
     if (mc != -INFINITY) l += p.pl[(base + c) * 16 + col] * fast_exp2(mc - m);
   }
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float acc = 0.f;
-    for (int c = 0; c < p.n_chunks; c++) {
-      const float mc = p.pm[(base + c) * 16 + col];
-      if (mc != -INFINITY) acc += p.po[((base + c) * 16 + col) * D + d] * fast_exp2(mc - m);
-    }
-    o[(long long)b * osb + (long long)hq_all * osh + d] = (T)(l > 0.f ? acc / l : 0.f);
+  red[tid] = l;
+  __syncthreads();
+  for (int s = nt / 2; s > 0; s >>= 1) {
+    if (tid < s) red[tid] += red[tid + s];
+    __syncthreads();
   }
-  if (lse && threadIdx.x == 0) lse[(long long)b * p.Hkv * p.G + hq_all] = l > 0.f ? m + fast_log2(l) : INFINITY;
+  l = red[0];
+  float acc = 0.f;  // this thread's output column d = tid (nt >= D is guaranteed by the launch)
+  for (int c0 = 0; c0 < p.n_chunks; c0 += WCAP) {
+    const int n = min(WCAP, p.n_chunks - c0);
+    __syncthreads();
+    for (int c = tid; c < n; c += nt) {
+      const float mc = p.pm[(base + c0 + c) * 16 + col];
+      w_s[c] = mc != -INFINITY ? fast_exp2(mc - m) : 0.f;
+    }
+    __syncthreads();
+    if (tid < D) {
+#pragma unroll 4
+      for (int c = 0; c < n; c++) acc += p.po[((base + c0 + c) * 16 + col) * D + tid] * w_s[c];
+    }
+  }
+  if (tid < D) o[(long long)b * osb + (long long)hq_all * osh + tid] = (T)(l > 0.f ? acc / l : 0.f);
+  if (lse && tid == 0) lse[(long long)b * p.Hkv * p.G + hq_all] = l > 0.f ? m + fast_log2(l) : INFINITY;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -172,8 +198,6 @@ __global__ __launch_bounds__(256) void decode_score_select_kernel(ScoreParams p)
   using v8 = typename E::v8;
   constexpr int NK = D / 32;
   __shared__ float bscore[MAX_SCORE_BLOCKS];
-  __shared__ float red_v[256];
-  __shared__ int red_i[256];
   __shared__ int picked[64];
   const int h = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
@@ -223,7 +247,9 @@ __global__ __launch_bounds__(256) void decode_score_select_kernel(ScoreParams p)
     bscore[blk] = v;
   }
   __syncthreads();
-  // phase C: k_out rounds of (largest value, smallest index)
+  // phase C: k_out rounds of (largest value, smallest index): wave-wide maxima of 64-bit (score, -index) keys,
+  // then the four wave results through LDS
+  __shared__ long long wave_best[4];
   for (int round = 0; round < p.k_out; round++) {
     float bv = -1.f;
     int bi = 0x7fffffff;
@@ -231,16 +257,16 @@ __global__ __launch_bounds__(256) void decode_score_select_kernel(ScoreParams p)
       const float v = bscore[blk];
       if (v > bv) { bv = v; bi = blk; }
     }
-    red_v[tid] = bv; red_i[tid] = bi;
+    const long long best = wave_max_i64(candidate_key(bv, bi));
+    if (lane == 0) wave_best[wave] = best;
     __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-      if (tid < s) {
-        const float ov = red_v[tid + s]; const int oi = red_i[tid + s];
-        if (ov > red_v[tid] || (ov == red_v[tid] && oi < red_i[tid])) { red_v[tid] = ov; red_i[tid] = oi; }
-      }
-      __syncthreads();
+    if (tid == 0) {
+      long long m = wave_best[0];
+      for (int w = 1; w < 4; w++) m = wave_best[w] > m ? wave_best[w] : m;
+      const int win = candidate_index(m);
+      picked[round] = win;
+      bscore[win] = -2.f;
     }
-    if (tid == 0) { picked[round] = red_i[0]; bscore[red_i[0]] = -2.f; }
     __syncthreads();
   }
   // ascending order, ids beyond the query's block become -1 at the tail
