@@ -108,11 +108,14 @@ int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* dx, void* d
 /* ---- linear_compress ----------------------------------------------------------------------------
  * Forward: replaces linear_compress_fwd_kernel (native_sparse_attention/ops/triton/linear_compress.py:27-136,
  * launched at :379-410).  x [total_x,H,D]; w [H, kernel_size*D, D] contiguous; y [total_y,H,D].
+ * workspace (16-byte aligned; may be NULL when the size query returns 0): fp32 partials of the split contraction.
  */
+size_t nsa_linear_compress_fwd_workspace_bytes(int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim, int64_t kernel_size);
 int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
                             int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
                             int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
-                            int64_t y_stride_n, int64_t y_stride_h, int dtype, void* stream);
+                            int64_t y_stride_n, int64_t y_stride_h, int dtype, void* workspace, size_t workspace_bytes,
+                            void* stream);
 /* Backward: replaces linear_compress_bwd_kernel and its fp32 atomic adds (:140-306, launched at
  * :449-480).  dx [total_x,H,D]; dw [H, kernel_size*D, D] contiguous, both in the dtype of x.
  * Gather formulation, no atomics: reproducible.

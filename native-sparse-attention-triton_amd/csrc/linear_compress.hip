@@ -13,6 +13,7 @@ struct LinParams {
   const int32_t* cu; const int32_t* ycu;
   int total_x, total_y, batch, H, ks, st;
   long long xsn, xsh, ysn, ysh, dysn, dysh, dxsn, dxsh;  // w, dw: [H, ks*D, D] contiguous
+  float* partial; int splits;                            // forward split over the contraction: fp32 [splits][total_y][H][D]
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -84,11 +85,15 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(LinParams p) {
       if (pc < PIECES) *reinterpret_cast<uint4*>(&w_s[buf][pc / (D / 8)][(pc % (D / 8)) * 8]) = regs[u];
     }
   };
-  const int n_steps = p.ks * NK;  // step = (k, 32-wide slice of d): rows [32*step, +32) of W[h]
-  fetch(0);
-  stash(0);
+  // step = (k, 32-wide slice of d): rows [32*step, +32) of W[h]; blockIdx.z takes a contiguous share of the steps
+  const int all_steps = p.ks * NK, per = (all_steps + p.splits - 1) / p.splits;
+  const int step0 = blockIdx.z * per, n_steps = min(all_steps, step0 + per);
+  if (step0 < n_steps) {
+    fetch(step0);
+    stash(step0 & 1);
+  }
   __syncthreads();
-  for (int step = 0; step < n_steps; step++) {
+  for (int step = step0; step < n_steps; step++) {
     const int buf = step & 1;
     if (step + 1 < n_steps) fetch(step + 1);
     const int k = step / NK, c = step % NK;
@@ -98,7 +103,7 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(LinParams p) {
     if (step + 1 < n_steps) stash(buf ^ 1);
     __syncthreads();
   }
-  if (live) {
+  if (live && p.splits == 1) {
     T* yp = (T*)p.y + (long long)(p.ycu[b] + n) * p.ysn + (long long)h * p.ysh + 4 * lg;
 #pragma unroll
     for (int et = 0; et < NET; et++) {
@@ -107,7 +112,28 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(LinParams p) {
       for (int r = 0; r < 4; r++) o[r] = (T)acc[et][r];
       st8(yp + 16 * et, o);
     }
+  } else if (live) {
+    float* pp = p.partial + (((long long)blockIdx.z * p.total_y + p.ycu[b] + n) * p.H + h) * D + 4 * lg;
+#pragma unroll
+    for (int et = 0; et < NET; et++) *reinterpret_cast<f32x4*>(pp + 16 * et) = acc[et];
   }
+}
+
+// y = sum over the splits of the fp32 partials, in a fixed order
+template <typename T, int D>
+__global__ __launch_bounds__(256) void lin_reduce_kernel(LinParams p) {
+  using v4 = typename Elem<T>::v4;
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // (row, head, 4-wide piece)
+  const long long n_pieces = (long long)p.total_y * p.H * (D / 4);
+  if (i >= n_pieces) return;
+  const int c = (int)(i % (D / 4)), h = (int)((i / (D / 4)) % p.H);
+  const long long row = i / ((long long)(D / 4) * p.H);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < p.splits; z++) acc += *reinterpret_cast<const f32x4*>(p.partial + (long long)z * p.total_y * p.H * D + i * 4);
+  v4 o;
+#pragma unroll
+  for (int r = 0; r < 4; r++) o[r] = (T)acc[r];
+  st8((T*)p.y + row * p.ysn + (long long)h * p.ysh + 4 * c, o);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -242,7 +268,10 @@ template <typename T, int D>
 static int lin_run(const LinParams& p, int what, hipStream_t s) {
   if (what == 0) {
     const int64_t slots = p.total_y / 64 + p.batch + 1;
-    if (p.total_y > 0) lin_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)p.H), 256, 0, s>>>(p);
+    if (p.total_y > 0) {
+      lin_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)p.H, (unsigned)p.splits), 256, 0, s>>>(p);
+      if (p.splits > 1) lin_reduce_kernel<T, D><<<(unsigned)(((long long)p.total_y * p.H * (D / 4) + 255) / 256), 256, 0, s>>>(p);
+    }
   } else {
     const int64_t unit = 64 * (int64_t)p.st;
     const int64_t slots = p.total_x / unit + p.batch + 1;
@@ -273,18 +302,41 @@ static int lin_fill(LinParams& p, const void* x, const void* w, const int32_t* c
   p.x = x; p.w = w; p.cu = cu; p.ycu = ycu; p.total_x = (int)total_x; p.total_y = (int)total_y; p.batch = (int)batch; p.H = (int)H;
   p.ks = (int)ks; p.st = (int)st; p.xsn = xsn; p.xsh = xsh;
   p.dy = nullptr; p.y = nullptr; p.dx = nullptr; p.dw = nullptr; p.ysn = p.ysh = p.dysn = p.dysh = p.dxsn = p.dxsh = 0;
+  p.partial = nullptr; p.splits = 1;
   return NSA_OK;
+}
+
+// The forward has 64 output rows x one head per workgroup and kernel_size * D / 32 dependent steps: a few dozen
+// workgroups for a typical input.  The contraction is therefore split over up to 16 workgroups (fp32 partials,
+// summed in a fixed order) until about a thousand workgroups are in flight.
+static int lin_fwd_splits(int64_t total_y, int64_t batch, int64_t H, int64_t ks, int64_t head_dim) {
+  const int64_t wgs = (total_y / 64 + batch + 1) * H, steps = ks * (head_dim / 32);
+  int splits = 1;
+  while (splits < 16 && wgs * splits < 1024 && steps / (splits * 2) >= 4) splits *= 2;
+  return splits;
+}
+
+extern "C" size_t nsa_linear_compress_fwd_workspace_bytes(int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim, int64_t kernel_size) {
+  const int splits = lin_fwd_splits(total_y, batch, num_heads, kernel_size, head_dim);
+  return splits > 1 ? (size_t)splits * total_y * num_heads * head_dim * 4 : 0;
 }
 
 extern "C" int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
                                        int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
                                        int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
-                                       int64_t y_stride_n, int64_t y_stride_h, int dtype, void* stream) {
+                                       int64_t y_stride_n, int64_t y_stride_h, int dtype, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
   LinParams p;
   int rc = lin_fill(p, x, w, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, kernel_size, kernel_stride, x_stride_n, x_stride_h, dtype);
   if (rc != NSA_OK) return rc;
   if (total_y > 0 && (!y || (y_stride_n | y_stride_h) % 4 != 0 || (uintptr_t)y % 8 != 0)) return NSA_ERR_UNSUPPORTED;
   p.y = y; p.ysn = y_stride_n; p.ysh = y_stride_h;
+  p.splits = lin_fwd_splits(total_y, batch, num_heads, kernel_size, head_dim);
+  if (p.splits > 1) {
+    if (!workspace || (uintptr_t)workspace % 16 != 0) return NSA_ERR_BAD_ARG;
+    if (workspace_bytes < nsa_linear_compress_fwd_workspace_bytes(total_y, batch, num_heads, head_dim, kernel_size)) return NSA_ERR_WORKSPACE;
+    p.partial = (float*)workspace;
+  }
   return lin_dispatch(p, 0, head_dim, dtype, (hipStream_t)stream);
 }
 

@@ -36,7 +36,8 @@ _SIGNATURES = {
     "nsa_cmp_attn_select": (c_int, [P] * 6 + [I] * 13 + [P, F, c_int, P]),
     "nsa_cmp_attn_bwd_workspace_bytes": (Z, [I] * 6),
     "nsa_cmp_attn_bwd": (c_int, [P] * 11 + [I] * 8 + [P, F, c_int, P, Z, P]),
-    "nsa_linear_compress_fwd": (c_int, [P] * 5 + [I] * 11 + [c_int, P]),
+    "nsa_linear_compress_fwd_workspace_bytes": (Z, [I] * 5),
+    "nsa_linear_compress_fwd": (c_int, [P] * 5 + [I] * 11 + [c_int, P, Z, P]),
     "nsa_linear_compress_bwd": (c_int, [P] * 7 + [I] * 13 + [c_int, P]),
     "nsa_window_attn_fwd": (c_int, [P] * 6 + [I] * 6 + [P, F, c_int, P]),
     "nsa_cache_fill": (c_int, [P] * 7 + [I] * 10 + [P]),

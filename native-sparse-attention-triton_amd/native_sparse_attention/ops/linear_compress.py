@@ -29,10 +29,11 @@ class LinearCompress(torch.autograd.Function):
         total_y = int(y_cu_seqlens[-1]) if known_total is None else int(known_total)
         y = torch.empty(total_y, num_heads, head_dim, dtype=x.dtype, device=x.device)
         lib = _lib.load()
+        ws = _lib.workspace(lib.nsa_linear_compress_fwd_workspace_bytes(total_y, batch, num_heads, head_dim, kernel_size), x.device)
         rc = lib.nsa_linear_compress_fwd(
             x.data_ptr(), w.data_ptr(), y.data_ptr(), cu_seqlens.data_ptr(), y_cu_seqlens.data_ptr(), total_len, total_y,
             batch, num_heads, head_dim, kernel_size, kernel_stride, x.stride(0), x.stride(1), y.stride(0), y.stride(1),
-            _lib.dtype_code(x), _lib.stream_ptr(x))
+            _lib.dtype_code(x), ws.data_ptr(), ws.numel(), _lib.stream_ptr(x))
         _lib.check(rc, "nsa_linear_compress_fwd")
         ctx.save_for_backward(x, w, cu_seqlens, y_cu_seqlens)
         ctx.kernel_size, ctx.kernel_stride, ctx.total_y = kernel_size, kernel_stride, total_y
