@@ -739,6 +739,7 @@ static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, c
                       int dtype, void* stream) {
   if (!q || !k || !cu_q || !cu_k || !strides || Tq <= 0 || Tk < 0 || B <= 0 || Hkv <= 0 || Hq % Hkv != 0 || ks <= 0 || st <= 0) return NSA_ERR_BAD_ARG;
   if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  if (!(sm_scale > 0.f)) return NSA_ERR_UNSUPPORTED;  // running maxima are taken on unscaled scores
   for (int i = 0; i < 6; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 != 0) return NSA_ERR_UNSUPPORTED;
   CmpParams& p = a.p;

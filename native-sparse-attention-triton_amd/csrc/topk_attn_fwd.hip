@@ -215,6 +215,7 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   if (!q || !k || !v || !topk_idx || !o || !lse || !cu_seqlens || !workspace) return NSA_ERR_BAD_ARG;
   if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
   if (total_len >= (1ll << 31)) return NSA_ERR_BAD_ARG;
+  if (!(sm_scale > 0.f)) return NSA_ERR_UNSUPPORTED;  // running maxima are taken on unscaled scores
   // 16-byte fragment loads need 8-element alignment of every row start
   if ((q_stride_n | q_stride_h | k_stride_n | k_stride_h | v_stride_n | v_stride_h) % 8 != 0) return NSA_ERR_UNSUPPORTED;
   if ((o_stride_n | o_stride_h) % 4 != 0) return NSA_ERR_UNSUPPORTED;

@@ -40,3 +40,19 @@ def test_bad_arguments_are_rejected_without_launching():
     assert rc == -1
     rc = lib.nsa_dense_decode(None, None, None, None, None, 1, 16, 1, 128, 64, None, 1.0, 0, None, 0, None)
     assert rc == -1
+
+
+def test_more_host_side_checks():
+    lib = _lib.load()
+    fake = 1 << 20  # non-null, 16-byte aligned; never dereferenced: the checks below fail before any launch
+    # non-positive softmax scale is refused by the training/prefill attention entry points
+    rc = lib.nsa_topk_attn_fwd(fake, fake, fake, fake, fake, fake, fake, 128, 1, 16, 1, 128, 4, 64, 2048, 128, 128, 128, 128, 128,
+                               512, 4, 1, 2048, 128, -0.1, 0, fake, 1 << 30, 3, None)
+    assert rc == -2
+    # the split of the linear_compress forward: cfg1 shape (1021 outputs, 4 heads, kernel 32, d 128) -> 16 splits of fp32 partials
+    assert lib.nsa_linear_compress_fwd_workspace_bytes(1021, 3, 4, 128, 32) == 16 * 1021 * 4 * 128 * 4
+    assert lib.nsa_linear_compress_fwd_workspace_bytes(200000, 1, 8, 128, 32) == 0          # enough workgroups already
+    # a cache update with more sequences than the slab holds
+    assert lib.nsa_cache_stage_token(fake, fake, fake, fake, 5, 2, 128, 256, 128, 256, 128, 4, 32, 16, None) == -1
+    # rope needs row strides that are multiples of 8 elements
+    assert lib.nsa_rope(fake, fake, fake, fake, 10, 1, 2, 128, 260, 128, 256, 128, 0, 1, 1.0, 0, 0, None) == -2
