@@ -242,6 +242,11 @@ int nsa_cache_fill(const void* key, const void* value, const int32_t* cu_src, co
 int nsa_cache_stage_token(const void* key, const void* value, void* stage_slab, int32_t* stage_len, int64_t batch,
                           int64_t num_kv_heads, int64_t head_dim, int64_t k_stride_b, int64_t k_stride_h, int64_t v_stride_b,
                           int64_t v_stride_h, int64_t max_batch, int64_t kernel_size, int64_t kernel_stride, void* stream);
+/* Plain KV cache (KVCache.update_kv of module/kv_cache.py:56-122): the new token of sequence b goes to row
+ * slab_len[b] of slab[:, b], slab_len[b] += 1 (nothing is written once a sequence fills its rows). */
+int nsa_cache_append_token(const void* key, const void* value, void* slab, int32_t* slab_len, int64_t batch, int64_t num_kv_heads,
+                           int64_t head_dim, int64_t k_stride_b, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_h,
+                           int64_t max_batch, int64_t slab_rows, void* stream);
 int nsa_cache_commit_token(const void* const* tokens, const int64_t* strides, const int32_t* stage_len, void* compress_slab,
                            int32_t* compress_len, void* sparse_slab, int32_t* sparse_len, void* sliding_slab, int32_t* sliding_len,
                            int64_t batch, int64_t num_kv_heads, int64_t head_dim, int64_t max_batch, int64_t kernel_size,

@@ -110,6 +110,25 @@ __global__ __launch_bounds__(256) void cache_commit_kernel(CommitParams p) {
   }
 }
 
+struct AppendParams {
+  const u16* key; const u16* value; u16* slab; int32_t* len;
+  int H, D, max_batch, rows;
+  long long ksn, ksh, vsn, vsh;
+};
+
+// plain KV cache: the new token of every sequence goes to row len[b], len[b] += 1
+__global__ __launch_bounds__(256) void cache_append_kernel(AppendParams p) {
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const long long HD = (long long)p.H * p.D;
+  const int n = p.len[b];
+  __syncthreads();  // every wave holds the old length before thread 0 stores the new one
+  if (n >= p.rows) return;
+  const long long row = ((long long)b * p.rows + n) * HD, kv = (long long)p.max_batch * p.rows * HD;
+  copy_row(p.slab + row, p.key + (long long)b * p.ksn, p.ksh, p.H, p.D, tid, 256);
+  copy_row(p.slab + kv + row, p.value + (long long)b * p.vsn, p.vsh, p.H, p.D, tid, 256);
+  if (tid == 0) p.len[b] = n + 1;
+}
+
 static bool rows_ok(const void* ptr, int64_t sn, int64_t sh) { return ptr && (uintptr_t)ptr % 16 == 0 && sn % 8 == 0 && sh % 8 == 0; }
 
 extern "C" int nsa_cache_fill(const void* key, const void* value, const int32_t* cu_src, const int32_t* row_begin, const int32_t* row_end,
@@ -159,5 +178,18 @@ extern "C" int nsa_cache_commit_token(const void* const* tokens, const int64_t* 
   p.H = (int)num_kv_heads; p.D = (int)head_dim; p.max_batch = (int)max_batch; p.ks = (int)kernel_size; p.cmp_rows = (int)compress_rows;
   p.full_rows = (int)sparse_rows; p.window = (int)window_size;
   cache_commit_kernel<<<(unsigned)batch, 256, 0, (hipStream_t)stream>>>(p);
+  return nsa_check_launch();
+}
+
+extern "C" int nsa_cache_append_token(const void* key, const void* value, void* slab, int32_t* slab_len, int64_t batch, int64_t num_kv_heads,
+                                      int64_t head_dim, int64_t k_stride_b, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_h,
+                                      int64_t max_batch, int64_t slab_rows, void* stream) {
+  if (!slab || !slab_len || batch <= 0 || batch > max_batch || num_kv_heads <= 0 || slab_rows <= 0) return NSA_ERR_BAD_ARG;
+  if (head_dim % 8 != 0 || (uintptr_t)slab % 16 != 0 || !rows_ok(key, k_stride_b, k_stride_h) || !rows_ok(value, v_stride_b, v_stride_h)) return NSA_ERR_UNSUPPORTED;
+  AppendParams p;
+  p.key = (const u16*)key; p.value = (const u16*)value; p.slab = (u16*)slab; p.len = slab_len;
+  p.H = (int)num_kv_heads; p.D = (int)head_dim; p.max_batch = (int)max_batch; p.rows = (int)slab_rows;
+  p.ksn = k_stride_b; p.ksh = k_stride_h; p.vsn = v_stride_b; p.vsh = v_stride_h;
+  cache_append_kernel<<<(unsigned)batch, 256, 0, (hipStream_t)stream>>>(p);
   return nsa_check_launch();
 }

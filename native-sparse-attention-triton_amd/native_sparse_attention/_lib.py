@@ -41,6 +41,7 @@ _SIGNATURES = {
     "nsa_linear_compress_bwd": (c_int, [P] * 7 + [I] * 13 + [c_int, P]),
     "nsa_window_attn_fwd": (c_int, [P] * 6 + [I] * 6 + [P, F, c_int, P]),
     "nsa_cache_fill": (c_int, [P] * 7 + [I] * 10 + [P]),
+    "nsa_cache_append_token": (c_int, [P] * 4 + [I] * 9 + [P]),
     "nsa_cache_stage_token": (c_int, [P] * 4 + [I] * 10 + [P]),
     "nsa_cache_commit_token": (c_int, [P] * 9 + [I] * 8 + [P]),
     "nsa_gate_combine": (c_int, [P] * 5 + [I] * 3 + [P, c_int, P]),

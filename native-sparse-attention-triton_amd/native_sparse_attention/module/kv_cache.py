@@ -26,6 +26,44 @@ from .. import _lib
 from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
 
 
+class KVCache:
+    """Plain per-sequence KV cache for dense attention: slab [2, max_batch, max_length, num_kv_heads, head_dim] plus
+    an int32 length per sequence (counterpart of kv_cache.py:21-122 of the reference).  Both updates are one kernel
+    each and the lengths stay on the device."""
+
+    def __init__(self, max_batch_size: int, max_length: int, num_kv_heads: int, head_dim: int, dtype: torch.dtype,
+                 device: Union[str, torch.device] = "cuda"):
+        assert dtype in (torch.bfloat16, torch.float16) and head_dim % 8 == 0
+        self.max_batch_size, self.max_length = max_batch_size, max_length
+        self.num_kv_heads, self.head_dim, self.dtype, self.device = num_kv_heads, head_dim, dtype, device
+        self.kv_cache = torch.zeros(2, max_batch_size, max_length, num_kv_heads, head_dim, dtype=dtype, device=device)
+        self.kv_len = torch.zeros(max_batch_size, dtype=torch.int32, device=device)
+
+    def reset(self):
+        self.kv_len.zero_()  # rows beyond a length are never read
+
+    def update_kv(self, cu_seqlens: torch.Tensor, step: int, key: torch.Tensor, value: torch.Tensor):
+        assert key.shape == value.shape and key.shape[1:] == (self.num_kv_heads, self.head_dim) and key.dtype == self.dtype
+        batch = cu_seqlens.shape[0] - 1
+        assert batch <= self.max_batch_size
+        key, value = last_dim_contiguous(key), last_dim_contiguous(value)
+        lib = _lib.load()
+        if step == 0:
+            cu_seqlens = cu_seqlens.to(torch.int32).contiguous()
+            begin, end = cu_seqlens[:-1], cu_seqlens[1:]  # views into cu_seqlens, alive for the call
+            rc = lib.nsa_cache_fill(key.data_ptr(), value.data_ptr(), cu_seqlens.data_ptr(), begin.data_ptr(),
+                                    end.data_ptr(), self.kv_cache.data_ptr(), self.kv_len.data_ptr(), key.shape[0],
+                                    batch, self.num_kv_heads, self.head_dim, key.stride(0), key.stride(1), value.stride(0),
+                                    value.stride(1), self.max_batch_size, self.max_length, _lib.stream_ptr(key))
+            _lib.check(rc, "nsa_cache_fill")
+        else:
+            assert key.shape[0] == batch
+            rc = lib.nsa_cache_append_token(key.data_ptr(), value.data_ptr(), self.kv_cache.data_ptr(), self.kv_len.data_ptr(), batch,
+                                            self.num_kv_heads, self.head_dim, key.stride(0), key.stride(1), value.stride(0),
+                                            value.stride(1), self.max_batch_size, self.max_length, _lib.stream_ptr(key))
+            _lib.check(rc, "nsa_cache_append_token")
+
+
 class NSACache:
     def __init__(self, max_batch_size: int, max_length: int, num_kv_heads: int, head_dim: int, kernel_size: int,
                  kernel_stride: int, window_size: int, dtype: torch.dtype, device: Union[str, torch.device] = "cuda"):

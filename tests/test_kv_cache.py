@@ -165,3 +165,34 @@ def test_prefill_and_decode_updates(device, lens, steps, ks, st, window):
         for c in (mine, ref):
             c.update_kv(cu, step, ck1, cv1, k1, v1, sk1, sv1)
         _same(mine, ref, B)
+
+
+def test_plain_kv_cache_prefill_and_decode(device):
+    """KVCache (dense baseline) against slice assignments: a prefill, three appended tokens, then a reset and a new prefill."""
+    from native_sparse_attention.module import KVCache
+    Hkv, d, maxB, maxL = 2, 64, 4, 300
+    cache = KVCache(maxB, maxL, Hkv, d, torch.bfloat16, device)
+    g = torch.Generator(device=device).manual_seed(3)
+    for lens in ([100, 1, 257], [40, 33]):
+        cu = cu_from_lens(lens, device)
+        B = len(lens)
+        want = torch.zeros(2, B, maxL, Hkv, d, dtype=torch.bfloat16, device=device)
+        kv = torch.randn(2, sum(lens), Hkv + 1, d, generator=g, device=device).bfloat16()
+        k, v = kv[0, :, :Hkv], kv[1, :, 1:]            # strided views
+        cache.reset()
+        cache.update_kv(cu, 0, k, v)
+        s0 = 0
+        for b, L in enumerate(lens):
+            want[0, b, :L], want[1, b, :L] = k[s0:s0 + L], v[s0:s0 + L]
+            s0 += L
+        cur = list(lens)
+        for step in range(1, 4):
+            nk = torch.randn(B, Hkv, d, generator=g, device=device).bfloat16()
+            nv = torch.randn(B, Hkv, d, generator=g, device=device).bfloat16()
+            cache.update_kv(cu, step, nk, nv)
+            for b in range(B):
+                want[0, b, cur[b]], want[1, b, cur[b]] = nk[b], nv[b]
+                cur[b] += 1
+        assert cache.kv_len[:B].tolist() == cur
+        for b in range(B):
+            assert torch.equal(cache.kv_cache[:, b, :cur[b]], want[:, b, :cur[b]]), b
