@@ -13,7 +13,6 @@ entry for the forward, 2.5x that for the backward (five matmuls).
 import argparse
 import json
 import os
-import statistics
 import sys
 import time
 
@@ -43,29 +42,32 @@ def _events_ms(fn, iters):
 
 
 def cpu_baseline():
-    """Oracle (pure PyTorch restatement) on the host cores: the reference's CPU-runnable case -
-    varlen [512, 1024, 512], 16 q heads / 1 kv head, d=64, block 64, top-8, fp32, forward."""
+    """Oracle (pure PyTorch restatement) on the host cores, on a bounded sample of the headline workload: the same
+    heads and selection (64 q / 4 kv heads, d=128, block 64, top-16, fp32) on one 4096-token sequence, forward +
+    backward; two runs of several seconds each, the faster one reported."""
     sys.path.insert(0, ROOT)
     import oracle
     from native_sparse_attention.testing import cu_from_lens, make_topk_idx
 
     torch.manual_seed(0)
-    cu = cu_from_lens([512, 1024, 512])
-    q, k, v = torch.randn(2048, 16, 64), torch.randn(2048, 1, 64), torch.randn(2048, 1, 64)
-    idx = make_topk_idx(cu, 64, 8, 1, seed=0, local_blocks=1)
-    flops = 4 * 64 * 64 * 16 * int((idx >= 0).sum())
-    oracle.topk_sparse_attention(q, k, v, idx, 64, cu)
+    n = 4096
+    cu = cu_from_lens([n])
+    q, k, v = (torch.randn(n, h, 128, requires_grad=True) for h in (64, 4, 4))
+    idx = make_topk_idx(cu, 64, 16, 4, seed=0, local_blocks=2)
+    do = torch.randn(n, 64, 128)
+    flops = 3.5 * 4 * 128 * 64 * 16 * int((idx >= 0).sum())
     times = []
-    t_end = time.perf_counter() + 15.0
-    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 50):
+    for _ in range(2):
         t0 = time.perf_counter()
-        oracle.topk_sparse_attention(q, k, v, idx, 64, cu)
+        oracle.topk_sparse_attention(q, k, v, idx, 64, cu).backward(do)
         times.append(time.perf_counter() - t0)
-    med = statistics.median(times)
+        q.grad = k.grad = v.grad = None
+    best = min(times)
     return {
-        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "ms": med * 1e3,
-        "sample": "oracle forward fp32, cu_seqlens=[0,512,1536,2048], 16q/1kv heads, d=64, block 64, top-8; median of %d runs" % len(times),
+        "value": flops / best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "ms": best * 1e3,
+        "sample": "oracle forward+backward fp32 on one 4096-token sequence of the headline shape (64q/4kv heads, d=128, block 64, "
+                  "top-16); best of 2 runs",
     }
 
 
