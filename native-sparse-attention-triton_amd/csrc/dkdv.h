@@ -56,20 +56,41 @@ struct DkdvParams {
   float qk_scale, sm_scale;
 };
 
+// Asynchronous copies from global memory straight into LDS (no registers in between): every lane
+// supplies its own source address, the 64 lanes of a wave fill 64 consecutive 16-byte (4-byte) pieces
+// starting at the wave-uniform LDS address.  Completion is counted by vmcnt like any other load.
+typedef __attribute__((address_space(3))) void* nsa_lds_ptr;
+__device__ __forceinline__ void dma16(const void* src, unsigned char* lds) { __builtin_amdgcn_global_load_lds(src, (nsa_lds_ptr)lds, 16, 0, 0); }
+__device__ __forceinline__ void dma4(const void* src, unsigned char* lds) { __builtin_amdgcn_global_load_lds(src, (nsa_lds_ptr)lds, 4, 0, 0); }
+// Workgroup barrier that lets the n youngest vector-memory operations of each wave stay in flight: waits
+// for all LDS traffic and for all but n loads, then meets.  (__syncthreads() would wait for every
+// outstanding copy into LDS, including the ones meant to land during the next step.)
+template <int N> __device__ __forceinline__ void barrier_keeping_loads() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));  // vmcnt(N), lgkmcnt(0), expcnt untouched
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // GT1: the GQA group has at most 16 query heads (one head tile), which removes every run-time division
 template <typename T, int D, int BS, bool RANGE, bool GT1>
-__global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_kernel(DkdvParams p) {
+__global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 3 : 1) void dkdv_kernel(DkdvParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16;
   constexpr int NW = dkdv_waves(BS);          // waves per workgroup
   constexpr int KT = NSUB / NW;               // 16-key tiles per wave
   constexpr int NT = NW * 64;
-  constexpr int LD = lds_pitch(D);                   // padded LDS row (elements)
-  __shared__ __attribute__((aligned(16))) T q_s[2][2][16][LD];
-  __shared__ __attribute__((aligned(16))) T do_s[2][2][16][LD];
-  __shared__ __attribute__((aligned(16))) float lse_s[2][32], delta_s[2][32];
-  __shared__ int pos_s[2][2];
+  // Staged rows (2 row groups x 16 heads of Q, the same of dO) are CP 16-byte pieces long and not padded:
+  // the copy engine writes whole 1 KiB stretches.  Piece c of row r sits at position (c + 2r) mod CP
+  // instead, which for CP = 16 gives every access the bank (address mod 256) it would have with a row
+  // pitch of 288 bytes: 16-byte row-fragment reads and the transposing 8-byte reads run at full rate.
+  constexpr int CP = D > 64 ? 16 : (D > 32 ? 8 : 4);
+  constexpr int TENSOR_BYTES = 32 * CP * 16;
+  constexpr int BUF_BYTES = 2 * TENSOR_BYTES + 256;   // Q rows | dO rows | 32 lse | 32 delta
+  // three buffers in rotation, each its own array so that the compiler can tell a copy in flight into
+  // one of them from reads of another
+  __shared__ __attribute__((aligned(256))) unsigned char buf0[BUF_BYTES], buf1[BUF_BYTES], buf2[BUF_BYTES];
 
   const int total_items = p.chunk_off[p.n_seg];
   const int item = blockIdx.x;
@@ -92,7 +113,7 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
   const int n_rg = n_tok * GT;                // row groups (token, head tile) in this chunk
   const int n_step = (n_rg + 1) / 2;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 15, lg = lane >> 4;
 
   // stationary operands: this wave's keys of K and V, B-operand layout (column = key)
@@ -112,80 +133,59 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
 #pragma unroll
     for (int i = 0; i < NDT; i++) { dk[j][i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[j][i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
-  // staging: 2 row groups x 16 heads x D elements of Q and of dO per step, as 16-byte pieces.
-  // Q and dO are handled by separate, fully unrolled loops: selecting the tensor at run time makes
-  // the compiler fetch base pointers from a table and serialises the prefetch behind those loads.
-  constexpr int PIECES = 2 * 16 * (D / 8);       // per tensor
-  constexpr int PPT = (PIECES + NT - 1) / NT;
-  // token ids of this chunk, read once (list mode); every later global load then has a single
-  // level of dependence and can be issued two steps ahead
+  // token ids of this chunk, read once (list mode): the source addresses of a step then need no
+  // global load of their own
   __shared__ int tok_s[CHUNK_TOKENS];
   for (int i = tid; i < n_tok; i += NT) tok_s[i] = RANGE ? first + i : p.queries[first + i];
   __syncthreads();
-  // fetch() is branch-free: loads are always issued (from a clamped, valid address) and the
-  // validity mask is applied when the registers are written to LDS.  Conditional loads make the
-  // compiler wait for every outstanding load at each join, which defeats the prefetch.
-  struct Stage { uint4 qd[PPT]; uint4 dd[PPT]; float lse, delta; int pos; unsigned ok; };
-  Stage stg[2];
+
   const T* const qbase = (const T*)p.q + (long long)h * p.G * p.qsh;
   const T* const dbase = (const T*)p.dout + (long long)h * p.G * p.dsh;
   const float* const lbase = p.lse + (long long)h * p.G * p.total_len;
   const float* const ebase = p.delta + (long long)h * p.G * p.total_len;
 
-  auto fetch = [&](int step, Stage& sg) {
-    unsigned ok = 0;
+  constexpr int NI = CP / 2;                 // 1 KiB wave-copies per tensor per step
+  constexpr int LPW = (NI + NW - 1) / NW;    // of which one wave issues at most this many
+  constexpr int RPI = 64 / CP;               // rows per wave-copy
+  // copies per wave and step that every wave issues at least: waiting until no more than these are
+  // outstanding means that everything issued one step earlier has arrived
+  constexpr int KEEP = 2 * (NI / NW) + 1;
+  // Starts the copies of one step into `buf`.  Rows past the end of the chunk and heads past the group
+  // are read from clamped (valid) addresses; compute() gives them probability 0 by its own test.
+  auto issue = [&](int step, unsigned char* buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = min(tid + u * NT, PIECES - 1);
-      const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = pc / (D / 8) / 16;
-      const int r = step * 2 + rg;
-      const int rc = min(r, n_rg - 1);
-      const int t = tok_s[GT1 ? rc : rc / GT];
-      const int hq = (GT1 ? 0 : (rc % GT) * 16) + hd;
-      const int hc = min(hq, p.G - 1);
-      sg.qd[u] = *reinterpret_cast<const uint4*>(qbase + (long long)t * p.qsn + (long long)hc * p.qsh + 8 * c);
-      sg.dd[u] = *reinterpret_cast<const uint4*>(dbase + (long long)t * p.dsn + (long long)hc * p.dsh + 8 * c);
-      ok |= (unsigned)(r < n_rg && hq < p.G) << u;
+    for (int u = 0; u < LPW; u++) {
+      const int i = wave + NW * u;
+      if (NI % NW != 0 && i >= NI) break;
+      const int row = i * RPI + lane / CP;
+      const int c = ((lane % CP) - 2 * row) & (CP - 1);
+      const int cc = c < D / 8 ? c : D / 8 - 1;   // D = 96: four positions per row hold nothing
+      const int rg = row >> 4, hd = row & 15;
+      const int r = min(step * 2 + rg, n_rg - 1);
+      const int t = tok_s[GT1 ? r : r / GT];
+      const int hq = min((GT1 ? 0 : (r % GT) * 16) + hd, p.G - 1);
+      dma16(qbase + (long long)t * p.qsn + (long long)hq * p.qsh + 8 * cc, buf + i * 1024);
+      dma16(dbase + (long long)t * p.dsn + (long long)hq * p.dsh + 8 * cc, buf + TENSOR_BYTES + i * 1024);
     }
-    {
-      const int rg = (tid >> 4) & 1, hd = tid & 15;
-      const int r = step * 2 + rg;
-      const int rc = min(r, n_rg - 1);
-      const int t = tok_s[GT1 ? rc : rc / GT];
-      const int hq = (GT1 ? 0 : (rc % GT) * 16) + hd;
-      const int hc = min(hq, p.G - 1);
-      sg.lse = lbase[(long long)hc * p.total_len + t];
-      sg.delta = ebase[(long long)hc * p.total_len + t];
-      sg.pos = r < n_rg ? t - s0 : -1;
-      ok |= (unsigned)(r < n_rg && hq < p.G) << 31;
-    }
-    sg.ok = ok;
-  };
-  auto stash = [&](int buf, const Stage& sg) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * NT;
-      if (pc < PIECES) {
-        const int c = pc % (D / 8), hd = (pc / (D / 8)) % 16, rg = pc / (D / 8) / 16;
-        const unsigned m = 0u - ((sg.ok >> u) & 1u);  // all ones when the piece exists
-        uint4 a = sg.qd[u], b2 = sg.dd[u];
-        a.x &= m; a.y &= m; a.z &= m; a.w &= m;
-        b2.x &= m; b2.y &= m; b2.z &= m; b2.w &= m;
-        *reinterpret_cast<uint4*>(&q_s[buf][rg][hd][8 * c]) = a;
-        *reinterpret_cast<uint4*>(&do_s[buf][rg][hd][8 * c]) = b2;
-      }
-    }
-    if (tid < 32) {
-      const bool ok = sg.ok >> 31;
-      lse_s[buf][tid] = ok ? sg.lse : INFINITY;   // +inf -> probability 0 for rows that do not exist
-      delta_s[buf][tid] = ok ? sg.delta : 0.f;
-      if ((tid & 15) == 0) pos_s[buf][tid >> 4] = sg.pos;
+    {  // lanes 0..31: lse of the 32 rows, lanes 32..63: their delta (every wave writes the same 256 bytes:
+       // no wave-dependent branch, and the same number of copies in flight for all of them)
+      const int rg = (lane >> 4) & 1, hd = lane & 15;
+      const int r = min(step * 2 + rg, n_rg - 1);
+      const int t = tok_s[GT1 ? r : r / GT];
+      const int hq = min((GT1 ? 0 : (r % GT) * 16) + hd, p.G - 1);
+      dma4((lane < 32 ? lbase : ebase) + (long long)hq * p.total_len + t, buf + 2 * TENSOR_BYTES);
     }
   };
 
-  // one step of the pipeline with compile-time buffer / register-set roles (no run-time choice of
-  // the register set, which would force copies that wait for the loads in flight)
-  auto compute = [&](const int buf) {
+  auto compute = [&](int step, const unsigned char* buf) __attribute__((always_inline)) {
+    // position of the two tokens of this step and how many of their 16 rows are real heads
+    int pos[2], nh[2];
+#pragma unroll
+    for (int tk = 0; tk < 2; tk++) {
+      const int r = step * 2 + tk, rc = min(r, n_rg - 1);
+      pos[tk] = tok_s[GT1 ? rc : rc / GT] - s0;
+      nh[tk] = r < n_rg ? min(16, p.G - (GT1 ? 0 : (rc % GT) * 16)) : 0;
+    }
     // S = Q K^T and dP = dO V^T for this wave's keys; lane holds column key=li, rows 4*lg+r of each token
     v8 pf[KT], dsf[KT];
 #pragma unroll
@@ -196,22 +196,22 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < NK; kk++) {
-          v8 qa = ld16<v8>(&q_s[buf][tk][li][32 * kk + 8 * lg]);
-          v8 da = ld16<v8>(&do_s[buf][tk][li][32 * kk + 8 * lg]);
+          const int at = ((tk * 16 + li) * CP + ((4 * kk + lg + 2 * li) & (CP - 1))) * 16;
+          v8 qa = ld16<v8>(buf + at);
+          v8 da = ld16<v8>(buf + TENSOR_BYTES + at);
           s = E::mfma16(qa, kf[j][kk], s);
           dp = E::mfma16(da, vf[j][kk], dp);
         }
-        const int pos = pos_s[buf][tk];
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[buf][tk * 16 + 4 * lg]);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_s[buf][tk * 16 + 4 * lg]);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(buf + 2 * TENSOR_BYTES + (tk * 16 + 4 * lg) * 4);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(buf + 2 * TENSOR_BYTES + 128 + (tk * 16 + 4 * lg) * 4);
+        const bool seen = RANGE ? (key < len && (p.window == -2 || (key * p.st + p.ks - 1 <= pos[tk] && (p.window < 0 || key >= pos[tk] - p.window))))
+                                : key <= pos[tk];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float l2 = l4[r];
-          const float dl = d4[r];
-          const bool vis = RANGE ? (key < len && (p.window == -2 || (key * p.st + p.ks - 1 <= pos && (p.window < 0 || key >= pos - p.window)))) : key <= pos;
-          const float pr = fast_exp2(vis ? s[r] * p.qk_scale - l2 : -INFINITY);  // select, not a branch
+          const bool vis = seen && 4 * lg + r < nh[tk];
+          const float pr = fast_exp2(vis ? s[r] * p.qk_scale - l4[r] : -INFINITY);  // select, not a branch
           pf[j][tk * 4 + r] = (T)pr;
-          dsf[j][tk * 4 + r] = (T)(pr * (dp[r] - dl) * p.sm_scale);
+          dsf[j][tk * 4 + r] = (T)(pr * (dp[r] - d4[r]) * p.sm_scale);
         }
       }
     }
@@ -225,10 +225,10 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
       s16x8 qt, dot;
 #pragma unroll
       for (int tk = 0; tk < 2; tk++) {
-        const T* qa = &q_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
-        const T* da = &do_s[buf][tk][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
-        s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(qa));
-        s16x4 c = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(da));
+        const int row = tk * 16 + 4 * lg + (li >> 2);
+        const int at = (row * CP + ((2 * dt + ((li >> 1) & 1) + 2 * row) & (CP - 1))) * 16 + (li & 1) * 8;
+        s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(buf + at));
+        s16x4 c = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(buf + TENSOR_BYTES + at));
 #pragma unroll
         for (int r = 0; r < 4; r++) { qt[tk * 4 + r] = a[r]; dot[tk * 4 + r] = c[r]; }
       }
@@ -240,21 +240,25 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 2 : 1) void dkdv_ke
       }
     }
   };
-  auto pipeline_step = [&](int step, const int buf, Stage& refill, const Stage& ready) {
-    // `refill` was written to LDS one step ago: reuse it for step + 2 (clamped: the tail re-loads the last step)
-    fetch(min(step + 2, n_step - 1), refill);
-    compute(buf);
-    if (step + 1 < n_step) stash(buf ^ 1, ready);
-    __syncthreads();
+  // one step: start the copies for two steps ahead into the buffer that was read one step ago, work on
+  // the current buffer, then wait for the copies started one step ago (the next buffer) and meet
+  auto pipeline_step = [&](int step, const unsigned char* cur, unsigned char* refill) __attribute__((always_inline)) {
+    issue(step + 2, refill);   // steps past the end copy the last row again, harmlessly
+    compute(step, cur);
+    barrier_keeping_loads<KEEP>();
   };
-  fetch(0, stg[0]);
-  stash(0, stg[0]);
-  fetch(min(1, n_step - 1), stg[1]);
-  __syncthreads();
-  for (int step = 0; step < n_step; step += 2) {
-    pipeline_step(step, 0, stg[0], stg[1]);
-    if (step + 1 < n_step) pipeline_step(step + 1, 1, stg[1], stg[0]);
+  issue(0, buf0);
+  issue(1, buf1);
+  barrier_keeping_loads<KEEP>();
+  // three steps per trip so that the buffer roles are compile-time; a trip may run up to two steps past
+  // the end, which see no rows (nh = 0) and add nothing
+  for (int step = 0; step < n_step; step += 3) {
+    pipeline_step(step, buf0, buf2);
+    pipeline_step(step + 1, buf1, buf0);
+    pipeline_step(step + 2, buf2, buf1);
   }
+  // copies still in flight target LDS that the next workgroup on this CU may own: let them land first
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   // partial[item][0 = dK, 1 = dV][key][d], fp32
   float* out = p.partial + (long long)item * 2 * BS * D;
 #pragma unroll
