@@ -812,6 +812,7 @@ extern "C" int nsa_cmp_attn_bwd(const void* q, const void* k, const void* v, con
   if (workspace_bytes < nsa_cmp_attn_bwd_workspace_bytes(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
   a.o_in = o; a.p.dout = dout; a.p.lse = (float*)lse; a.p.dq = dq; a.dk = dk; a.dv = dv;
   a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
+  if (!dkdv_strides_fit(a.p.qsn, a.p.qsh, a.p.dsn, a.p.dsh, a.p.G, head_dim)) return NSA_ERR_UNSUPPORTED;
   a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
   a.ws = (char*)workspace;
   a.what = 2;
@@ -851,6 +852,7 @@ extern "C" int nsa_window_attn_bwd(const void* q, const void* k, const void* v, 
   if (workspace_bytes < nsa_window_attn_bwd_workspace_bytes(total_len, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
   a.o_in = o; a.p.dout = dout; a.p.lse = (float*)lse; a.p.dq = dq; a.dk = dk; a.dv = dv;
   a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
+  if (!dkdv_strides_fit(a.p.qsn, a.p.qsh, a.p.dsn, a.p.dsh, a.p.G, head_dim)) return NSA_ERR_UNSUPPORTED;
   a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
   a.p.window = (int)(window_size > (1 << 30) ? (1 << 30) : window_size);
   a.ws = (char*)workspace;
@@ -893,6 +895,7 @@ extern "C" int nsa_flash_attn_bwd(const void* q, const void* k, const void* v, c
   if (workspace_bytes < nsa_flash_attn_bwd_workspace_bytes(total_q, total_k, batch, num_q_heads, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
   a.o_in = o; a.p.dout = dout; a.p.lse = (float*)lse; a.p.dq = dq; a.dk = dk; a.dv = dv;
   a.p.osn = strides[6]; a.p.osh = strides[7]; a.p.dsn = strides[8]; a.p.dsh = strides[9];
+  if (!dkdv_strides_fit(a.p.qsn, a.p.qsh, a.p.dsn, a.p.dsh, a.p.G, head_dim)) return NSA_ERR_UNSUPPORTED;
   a.p.dqsn = strides[10]; a.p.dqsh = strides[11]; a.dksn = strides[12]; a.dksh = strides[13]; a.dvsn = strides[14]; a.dvsh = strides[15];
   a.p.window = causal ? (1 << 30) : -2;
   a.ws = (char*)workspace;

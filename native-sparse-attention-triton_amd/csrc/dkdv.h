@@ -15,9 +15,12 @@
 
 static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
 
-// Waves per dK/dV workgroup; each wave owns bs / (16 * waves) key tiles.  Every wave reads all
-// staged query rows from LDS, so fewer waves would mean fewer LDS reads per token, but two waves
-// of 32 keys need > 256 registers each (one wave per SIMD) and measured 17% slower than four.
+// Waves per dK/dV workgroup; each wave owns bs / (16 * waves) key tiles.  Every wave reads all staged
+// query rows from LDS, so fewer waves would mean fewer LDS reads per token, but 32 keys per wave need 192
+// registers for the stationary operands and the accumulators alone: at two waves per SIMD that spills,
+// and at one wave per SIMD (with the score and the dK/dV MFMAs of neighbouring steps interleaved by
+// hand) the single wave's instruction issue became the limit - both measured slower than one tile per
+// wave at three waves per SIMD.
 constexpr int dkdv_waves(int bs) { return bs >= 64 ? 4 : bs / 16; }
 
 // chunk_off = exclusive scan of ceil((seg_end - seg_begin)/CHUNK_TOKENS) over segments (single workgroup).
@@ -52,7 +55,7 @@ struct DkdvParams {
   int total_len, batch, Hkv, G, GT, max_blocks, n_seg, ks, st;
   int window;  // range mode: -1 compressed keys (key c seen from position c*st + ks - 1 on), >= 0 ordinary keys seen by [key, key + window], -2 every key seen by every position
   long long ksn, ksh, vsn, vsh;
-  int qsn, qsh, dsn, dsh;  // element strides of q / dO (checked on the host to fit 31 bits)
+  int qsn, qsh, dsn, dsh;  // element strides of q / dO (dkdv_strides_fit() on the host)
   float qk_scale, sm_scale;
 };
 
@@ -70,6 +73,13 @@ template <int N> __device__ __forceinline__ void barrier_keeping_loads() {
   __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));  // vmcnt(N), lgkmcnt(0), expcnt untouched
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+
+// Token and head strides of q / dO are carried as 32-bit numbers: they, and the offset of the last head of
+// a group, must fit 31 bits.
+static inline bool dkdv_strides_fit(long long qsn, long long qsh, long long dsn, long long dsh, long long G, long long D) {
+  const long long lim = 0x7fffffffLL;
+  return qsn >= 0 && dsn >= 0 && qsh >= 0 && dsh >= 0 && qsn <= lim && dsn <= lim && G * qsh + D <= lim && G * dsh + D <= lim;
 }
 
 // GT1: the GQA group has at most 16 query heads (one head tile), which removes every run-time division

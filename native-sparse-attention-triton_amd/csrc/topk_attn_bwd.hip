@@ -377,6 +377,7 @@ extern "C" int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, co
   a.osn = strides[6]; a.osh = strides[7]; a.dsn = strides[8]; a.dsh = strides[9];
   a.ish = strides[10]; a.isn = strides[11]; a.isk = strides[12];
   a.dqsn = strides[13]; a.dqsh = strides[14]; a.dksn = strides[15]; a.dksh = strides[16]; a.dvsn = strides[17]; a.dvsh = strides[18];
+  if (!dkdv_strides_fit(a.qsn, a.qsh, a.dsn, a.dsh, num_q_heads / num_kv_heads, head_dim)) return NSA_ERR_UNSUPPORTED;
   a.sm_scale = sm_scale; a.ws = (char*)workspace; a.stream = (hipStream_t)stream;
   a.out_seg_off = out_segment_offsets; a.out_queries = out_queries; a.phases = phases;
   if (dtype == NSA_BF16) return bwd_d<__bf16>(a);

@@ -56,3 +56,14 @@ def test_more_host_side_checks():
     assert lib.nsa_cache_stage_token(fake, fake, fake, fake, 5, 2, 128, 256, 128, 256, 128, 4, 32, 16, None) == -1
     # rope needs row strides that are multiples of 8 elements
     assert lib.nsa_rope(fake, fake, fake, fake, 10, 1, 2, 128, 260, 128, 256, 128, 0, 1, 1.0, 0, 0, None) == -2
+
+
+def test_backward_refuses_strides_beyond_31_bits():
+    lib = _lib.load()
+    fake = 1 << 20
+    # head stride of q times the group size must fit 31 bits for the dK/dV pass: [Hq, T, D] views of very long inputs do not
+    strides = (ctypes.c_int64 * 19)(128, 1 << 28, 512, 128, 512, 128, 8192, 128, 8192, 128, 2048 * 16, 16, 1, 8192, 128, 512, 128, 512, 128)
+    ws = lib.nsa_topk_attn_bwd_workspace_bytes(2048, 1, 64, 4, 128, 16, 64)
+    rc = lib.nsa_topk_attn_bwd(fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, 2048, 1, 64, 4, 128, 16, 64, strides, 0.1,
+                               0, fake, ws, None, None, 7, None)
+    assert rc == -2
