@@ -315,7 +315,10 @@ def main():
     bwd = lambda ph: _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_b, phases=ph, out=grads)
     kern = {
         "fwd_attend": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd),        # QK^T, PV
-        "bwd_prep": (_events_ms(lambda: bwd(1), it), 0.0),                  # delta + reverse index (HBM / integer)
+        # preparation run alone: delta pass + reverse index.  In a full backward the delta pass does not run (dQ
+        # forms delta from the dO rows it holds), so kernel_ms adds up to more than bwd_ms
+        "bwd_prep": (_events_ms(lambda: bwd(1), it), 0.0),
+        "bwd_index_and_dq": (_events_ms(lambda: bwd(5), it), 0.0),         # reverse index + dQ with delta formed inside
         "bwd_dkdv": (_events_ms(lambda: bwd(2), it), 2.0 * f_fwd),          # QK^T, dO V^T, P^T dO, dS^T Q
         "bwd_dq": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd),            # dS K (its recomputed QK^T, dO V^T are not counted)
     }

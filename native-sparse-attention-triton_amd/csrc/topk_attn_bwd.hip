@@ -106,11 +106,13 @@ __global__ __launch_bounds__(256) void segment_offsets_kernel(const uint32_t* __
 // ------------------------------------------------------------------------------------------
 // pass 4: dQ
 struct DqParams {
-  const void* q; const void* kf; const void* vf; const void* dout; const float* lse; const float* delta;
+  const void* q; const void* kf; const void* vf; const void* dout; const float* lse;
+  const void* o;   // forward output: when given, delta = rowsum(O * dO) is formed here and stored for the dK/dV pass
+  float* delta;    // read when o is null
   const int32_t* idx; const int32_t* cu; void* dq;
   int total_len, batch, Hkv, G, GT, topk, n_slots;
   long long n_items;
-  long long qsn, qsh, dsn, dsh, ish, isn, isk, dqsn, dqsh;
+  long long qsn, qsh, dsn, dsh, osn, osh, ish, isn, isk, dqsn, dqsh;
   float qk_scale, sm_scale;
 };
 
@@ -151,7 +153,22 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
     dof[kk] = has_head ? ld16<v8>(dp_ + 32 * kk) : zero16<v8>();
   }
   const float l2 = has_head ? p.lse[(long long)hh * p.total_len + t] : INFINITY;
-  const float dl = has_head ? p.delta[(long long)hh * p.total_len + t] : 0.f;
+  float dl;
+  if (p.o) {
+    // the wave holds this token's dO rows already: one more row of loads gives delta without a pass of its own
+    const T* op_ = (const T*)p.o + (long long)t * p.osn + (long long)hh * p.osh + 8 * lg;
+    float part = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) {
+      const v8 of = has_head ? ld16<v8>(op_ + 32 * kk) : zero16<v8>();
+#pragma unroll
+      for (int e = 0; e < 8; e++) part = __builtin_fmaf((float)of[e], (float)dof[kk][e], part);
+    }
+    dl = column_sum(part);
+    if (has_head && lg == 0) p.delta[(long long)hh * p.total_len + t] = dl;
+  } else {
+    dl = has_head ? p.delta[(long long)hh * p.total_len + t] : 0.f;
+  }
   f32x4 acc[NDT];
 #pragma unroll
   for (int i = 0; i < NDT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -282,7 +299,10 @@ static int run_bwd(const BwdArgs& a) {
   float* delta = (float*)(ws + L.delta);
   const int G = (int)(a.Hq / a.Hkv), GT = (G + 15) / 16;
   const int n_seg = (int)(a.Hkv * L.max_blocks);
-  if (a.phases & NSA_BWD_PHASE_PREP)
+  // delta = rowsum(O * dO): formed inside the dQ pass when that pass runs in the same call (it holds the dO
+  // rows anyway), by a pass of its own when only the preparation is asked for
+  const bool fused_delta = (a.phases & NSA_BWD_PHASE_PREP) && (a.phases & NSA_BWD_PHASE_DQ);
+  if ((a.phases & NSA_BWD_PHASE_PREP) && !fused_delta)
     launch_delta<T, D>((const T*)a.o, (const T*)a.dout, delta, a.T, a.Hq, a.osn, a.osh, a.dsn, a.dsh, a.stream);
   if (a.phases & NSA_BWD_PHASE_PREP) {
     int rc = build_reverse_index(a, L);
@@ -291,6 +311,22 @@ static int run_bwd(const BwdArgs& a) {
   if (a.out_seg_off) {
     (void)hipMemcpyAsync(a.out_seg_off, ws + L.seg_off, (size_t)(n_seg + 1) * 4, hipMemcpyDeviceToDevice, a.stream);
     (void)hipMemcpyAsync(a.out_queries, ws + L.vals_out, (size_t)L.n_pairs * 4, hipMemcpyDeviceToDevice, a.stream);
+  }
+  // dQ first: it leaves delta behind for the dK/dV pass
+  if (a.phases & NSA_BWD_PHASE_DQ) {
+    DqParams p;
+    T* kf = (T*)(ws + L.kf);
+    T* vf = (T*)(ws + L.vf);
+    launch_retile<T, D, RETILE_ROWS>((const T*)a.k, kf, a.cu, a.B, a.ksn, a.ksh, L.n_slots, a.Hkv, a.stream);
+    launch_retile<T, D, RETILE_ROWS>((const T*)a.v, vf, a.cu, a.B, a.vsn, a.vsh, L.n_slots, a.Hkv, a.stream);
+    p.q = a.q; p.kf = kf; p.vf = vf; p.dout = a.dout; p.lse = a.lse; p.o = fused_delta ? a.o : nullptr; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
+    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk; p.n_slots = (int)L.n_slots;
+    p.n_items = (long long)a.T * GT * a.Hkv;
+    p.qsn = a.qsn; p.qsh = a.qsh; p.dsn = a.dsn; p.dsh = a.dsh; p.osn = a.osn; p.osh = a.osh;
+    p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
+    p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
+    long long n_wg = ((p.n_items + 3) / 4 + 7) / 8 * 8;
+    dq_kernel<T, D, BS><<<(unsigned)n_wg, 256, 0, a.stream>>>(p);
   }
   if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;
@@ -306,21 +342,6 @@ static int run_bwd(const BwdArgs& a) {
     else dkdv_kernel<T, D, BS, false, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
     dkdv_reduce_kernel<T, D, BS><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(
         p.partial, p.chunk_off, a.cu, p.cu_blk, (int)a.B, (int)L.max_blocks, (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
-  }
-  if (a.phases & NSA_BWD_PHASE_DQ) {
-    DqParams p;
-    T* kf = (T*)(ws + L.kf);
-    T* vf = (T*)(ws + L.vf);
-    launch_retile<T, D, RETILE_ROWS>((const T*)a.k, kf, a.cu, a.B, a.ksn, a.ksh, L.n_slots, a.Hkv, a.stream);
-    launch_retile<T, D, RETILE_ROWS>((const T*)a.v, vf, a.cu, a.B, a.vsn, a.vsh, L.n_slots, a.Hkv, a.stream);
-    p.q = a.q; p.kf = kf; p.vf = vf; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
-    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk; p.n_slots = (int)L.n_slots;
-    p.n_items = (long long)a.T * GT * a.Hkv;
-    p.qsn = a.qsn; p.qsh = a.qsh; p.dsn = a.dsn; p.dsh = a.dsh;
-    p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
-    p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
-    long long n_wg = ((p.n_items + 3) / 4 + 7) / 8 * 8;
-    dq_kernel<T, D, BS><<<(unsigned)n_wg, 256, 0, a.stream>>>(p);
   }
   return nsa_check_launch();
 }
