@@ -70,6 +70,9 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
  * dK/dV are reduced in a fixed order (no atomics): results are run-to-run deterministic.
  * phases: NSA_BWD_PHASE_ALL, or a subset to re-run single passes on a workspace that an
  * earlier call with identical arguments has already filled (PREP = delta + reverse index).
+ * When PREP and DQ run in the same call, delta = rowsum(o * dout) is formed inside the dQ pass
+ * (which runs before dK/dV) instead of by a pass of its own; the stored values are the same.
+ * Token strides of q and dout, and group_size * their head strides + D, must fit 31 bits.
  */
 #define NSA_BWD_PHASE_PREP 1
 #define NSA_BWD_PHASE_DKDV 2
