@@ -79,7 +79,7 @@ def _time_ms(fn, iters, warm=2):
 
 
 def bench_pipeline(args, dev):
-    """BASELINE config 1: linear_compress -> compressed_attention (+selection) -> topk_sparse_attention, forward, bf16."""
+    """Pipeline benchmark: linear_compress -> compressed_attention (+selection) -> topk_sparse_attention, forward, bf16."""
     from native_sparse_attention.ops import compressed_attention, linear_compress, topk_sparse_attention
     from native_sparse_attention.ops.compressed_attention import _compressed_attention_fwd, _select_blocks
     from native_sparse_attention.testing import cu_from_lens
@@ -127,7 +127,7 @@ def bench_pipeline(args, dev):
 
 
 def bench_compressed(args, dev):
-    """BASELINE config 3: weightedpool compression + compressed_attention forward+backward, N=65536, 32q/2kv."""
+    """Long-sequence benchmark: weightedpool compression + compressed_attention forward+backward, N=65536, 32q/2kv."""
     from native_sparse_attention.ops import compressed_attention, weightedpool_compress
     from native_sparse_attention.ops.compressed_attention import _compressed_attention_bwd, _compressed_attention_fwd, _select_blocks
     from native_sparse_attention.testing import cu_from_lens
@@ -177,7 +177,7 @@ def bench_compressed(args, dev):
 
 
 def bench_decode(args, dev):
-    """BASELINE config 4: one NSA decode step over the cache slabs (three branches + sigmoid gates)."""
+    """Decode benchmark: one NSA decode step over the cache slabs (three branches + sigmoid gates)."""
     from native_sparse_attention.infer import nsa_infer
     from native_sparse_attention.module import NSACache
     from native_sparse_attention.ops import weightedpool_compress
@@ -262,7 +262,7 @@ def main():
     ap.add_argument("--readme-heads", action="store_true",
                     help="compressed workload with the 64q/4kv head layout of the reference README tables instead of config 3's 32q/2kv")
     ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode"],
-                    help="topk = the headline metric (default); the others time BASELINE configs 1, 3 and 4")
+                    help="topk = the headline metric (default); the others time the pipeline, long-sequence compressed-attention and decode benchmarks")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the operator path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)

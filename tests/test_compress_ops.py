@@ -82,7 +82,7 @@ def test_pool_asserts(device):
 
 LINEAR_CASES = [
     # lens, H, d, ks, st, dtype
-    ([1024, 7168, 8192], 4, 128, 32, 16, torch.bfloat16),         # BASELINE config 1 shape
+    ([1024, 7168, 8192], 4, 128, 32, 16, torch.bfloat16),         # pipeline benchmark shape
     ([12, 100, 257, 64], 2, 64, 32, 16, torch.float16),
     ([300, 75], 3, 96, 16, 16, torch.bfloat16),
     ([500], 2, 192, 32, 16, torch.float16),                        # the reference's d=192 smoke shape

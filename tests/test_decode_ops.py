@@ -37,7 +37,7 @@ def _decode_idx(lens, bs, topk, Hkv, device):
 
 @pytest.mark.parametrize("B,max_len,Hq,Hkv,d,dtype", [
     (76, 8192, 32, 4, 128, torch.float16),     # the reference's own check
-    (4, 512, 32, 2, 128, torch.bfloat16),      # sliding-window ring of BASELINE config 4
+    (4, 512, 32, 2, 128, torch.bfloat16),      # sliding-window ring of the decode benchmark
     (3, 200, 6, 2, 64, torch.bfloat16),        # G=3
     (2, 130, 40, 2, 96, torch.float16),        # G=20: two head tiles
 ])
@@ -51,7 +51,7 @@ def test_dense_decode(device, B, max_len, Hq, Hkv, d, dtype):
 
 @pytest.mark.parametrize("B,max_len,Hq,Hkv,d,bs,topk,dtype", [
     (76, 8192, 32, 4, 128, 64, 16, torch.float16),   # the reference's own check
-    (4, 8193, 32, 2, 128, 64, 8, torch.bfloat16),    # BASELINE config 4 sparse branch
+    (4, 8193, 32, 2, 128, 64, 8, torch.bfloat16),    # decode benchmark, sparse branch
     (5, 1000, 8, 2, 64, 32, 4, torch.bfloat16),
     (3, 1500, 16, 1, 128, 128, 3, torch.bfloat16),
     (3, 1500, 16, 1, 32, 256, 2, torch.float16),
@@ -70,7 +70,7 @@ def test_topk_decode(device, B, max_len, Hq, Hkv, d, bs, topk, dtype):
 
 
 @pytest.mark.parametrize("lens,Hq,Hkv,d,topk,dtype", [
-    ([2049, 4097, 6145, 8193], 32, 2, 128, 8, torch.bfloat16),   # BASELINE config 4 compressed branch
+    ([2049, 4097, 6145, 8193], 32, 2, 128, 8, torch.bfloat16),   # decode benchmark, compressed branch
     ([40, 100, 31, 700], 8, 2, 64, 16, torch.float16),           # one sequence without compressed tokens
     ([64, 65], 4, 1, 128, 4, torch.bfloat16),
 ])

@@ -1,4 +1,4 @@
-"""The headline configurations at full size (BASELINE configs 2 and 3) on the GPU, checked through properties that do
+"""The headline configurations at full size (the top-k sweep's N=32768 point and the N=65536 compressed-attention benchmark) on the GPU, checked through properties that do
 not need a dense oracle: sampled-row parity of the forward and of dQ (a row of either depends on that row's attention
 only), and exact identities of the backward:
   * every row of P sums to 1, so  sum_j dV[j, hkv, :] = sum_t sum_{h in group} dO[t, h, :]  (over rows that see a key);

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 CASES = [
     # lens, Hq, Hkv, d, block, topk, dtype, local_blocks
-    ([512, 1024, 512], 16, 1, 64, 64, 8, torch.bfloat16, 1),          # BASELINE config 0 shape
+    ([512, 1024, 512], 16, 1, 64, 64, 8, torch.bfloat16, 1),          # shape of the reference's CPU-runnable test
     ([1000, 2000, 4096], 64, 8, 96, 64, 5, torch.float16, 1),         # the reference's own test shape
     ([2048], 64, 4, 128, 64, 16, torch.bfloat16, 2),                  # sweep shape, small N
     ([4096], 64, 4, 128, 64, 8, torch.bfloat16, 2),
