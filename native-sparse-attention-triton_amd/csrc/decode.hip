@@ -17,17 +17,22 @@ struct DecodeParams {
   float qk_scale;
 };
 
-// MODE 0: dense prefix, MODE 1: top-k blocks
+// MODE 0: dense prefix, MODE 1: top-k blocks.  A wave owns one chunk of up to 64 keys and writes its own
+// partial: nothing is exchanged between the waves of a workgroup, so the kernel has no barrier.  The V rows
+// of the chunk are copied straight from global memory into a wave-private LDS tile (no registers, no
+// ds_write) while the scores are formed; rows are 256 bytes, unpadded, with the 16-byte pieces of row r
+// rotated by 2r positions so that the transposing reads hit every bank once.
 template <typename T, int D, int MODE>
 __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
-  constexpr int NK = D / 32, NDT = D / 16, LD = lds_pitch(D);
-  __shared__ __attribute__((aligned(16))) T v_s[4][16][LD];
-  __shared__ float m_s[4][16], l_s[4][16];
-  __shared__ float o_s[16][D + 1];
-  const int chunk = blockIdx.x, h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT, b = blockIdx.z;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  constexpr int NK = D / 32, NDT = D / 16;
+  constexpr int CP = D > 64 ? 16 : (D > 32 ? 8 : 4);   // 16-byte pieces per staged row
+  constexpr int RPI = 64 / CP;                         // rows per 1 KiB wave-copy
+  __shared__ __attribute__((aligned(256))) unsigned char v_s[4][64 * CP * 16];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, lg = lane >> 4;
+  const int chunk = blockIdx.x * 4 + wave, h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT, b = blockIdx.z;
+  if (chunk >= p.n_chunks) return;
   const int len = min(p.lens[b], p.slab_len);  // never read past the slab
   int k0, kend;  // keys [k0, kend) of this chunk are visible
   if (MODE == 0) {
@@ -46,137 +51,134 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
   float* pl = p.pl + slot * 16;
   float* po = p.po + slot * 16 * D;
   if (kend <= k0) {  // nothing visible: neutral partial
-    if (tid < 16) { pm[tid] = -INFINITY; pl[tid] = 0.f; }
-    for (int i = tid; i < 16 * D; i += 256) po[i] = 0.f;
+    if (lane < 16) { pm[lane] = -INFINITY; pl[lane] = 0.f; }
+    for (int i = lane; i < 16 * D; i += 64) po[i] = 0.f;
     return;
+  }
+  // V rows -> LDS, started first.  Rows past kend are copied from row k0 (slab rows past the length may hold
+  // anything, and 0 * NaN would poison the sum); their probabilities are exactly 0.
+  unsigned char* vs = v_s[wave];
+#pragma unroll
+  for (int i = 0; i < 64 / RPI; i++) {
+    const int row = i * RPI + lane / CP;
+    const int c = ((lane % CP) - 2 * row) & (CP - 1);
+    const int cc = c < D / 8 ? c : D / 8 - 1;
+    const int key = k0 + row < kend ? k0 + row : k0;
+    dma16((const T*)p.v + (long long)b * p.vsb + (long long)key * p.vsn + (long long)h * p.vsh + 8 * cc, vs + i * 1024);
   }
   const int hq = gt * 16 + li;
   const bool has_head = hq < p.G;
   const T* qp = (const T*)p.q + (long long)b * p.qsb + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
-  v8 qf[NK];
+  v8 qf[NK], kf[4][NK];
 #pragma unroll
   for (int kk = 0; kk < NK; kk++) qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
-  // this wave's 16 keys
-  const int kw = k0 + 16 * wave;
-  {
-    const int key = kw + li;
-    const int row = key < kend ? key : k0;
-    const T* kp = (const T*)p.k + (long long)b * p.ksb + (long long)row * p.ksn + (long long)h * p.ksh + 8 * lg;
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
-    if (kw < kend) {
 #pragma unroll
-      for (int kk = 0; kk < NK; kk++) s = E::mfma16(ld16<v8>(kp + 32 * kk), qf[kk], s);
-    }
-    // stage V rows (zeros for invisible keys: slab rows past the length may hold anything)
-    constexpr int PIECES = 16 * (D / 8);
-    for (int i = lane; i < PIECES; i += 64) {
-      const int r = i / (D / 8), c = (i % (D / 8)) * 8;
-      uint4 val = {0u, 0u, 0u, 0u};
-      if (kw + r < kend) val = *reinterpret_cast<const uint4*>((const T*)p.v + (long long)b * p.vsb + (long long)(kw + r) * p.vsn + (long long)h * p.vsh + c);
-      *reinterpret_cast<uint4*>(&v_s[wave][r][c]) = val;
-    }
-    float mw = -INFINITY;
+  for (int nt = 0; nt < 4; nt++) {
+    const int key = k0 + 16 * nt + li;
+    const T* kp = (const T*)p.k + (long long)b * p.ksb + (long long)(key < kend ? key : k0) * p.ksn + (long long)h * p.ksh + 8 * lg;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const float x = (kw + 4 * lg + r) < kend ? s[r] * p.qk_scale : -INFINITY;
-      s[r] = x;
-      mw = fmaxf(mw, x);
-    }
-    mw = column_max(mw);
-    float lw = 0.f;
-    v8 pf = zero16<v8>();
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const float x = mw == -INFINITY ? 0.f : fast_exp2(s[r] - mw);
-      lw += x;
-      pf[r] = (T)x;
-    }
-    lw = column_sum(lw);
-    if (lg == 0) { m_s[wave][li] = mw; l_s[wave][li] = lw; }
-    __syncthreads();  // v_s staged, m_s/l_s visible
-    float m = fmaxf(fmaxf(m_s[0][li], m_s[1][li]), fmaxf(m_s[2][li], m_s[3][li]));
-    const float sc = mw == -INFINITY ? 0.f : fast_exp2(mw - m);
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    f32x4 acc[NDT];
-#pragma unroll
-    for (int dt = 0; dt < NDT; dt++) {
-      const T* va = &v_s[wave][4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
-      s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(va));
-      s16x8 a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
-      f32x4 z = {0.f, 0.f, 0.f, 0.f};
-      acc[dt] = E::mfma16(__builtin_bit_cast(v8, a8), pf, z);
-    }
-    // o_s[head][d] = sum over waves of sc * acc, one wave at a time
-    for (int w = 0; w < 4; w++) {
-      if (wave == w) {
-#pragma unroll
-        for (int dt = 0; dt < NDT; dt++)
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            float* dst = &o_s[li][16 * dt + 4 * lg + r];
-            *dst = (w == 0 ? 0.f : *dst) + sc * acc[dt][r];
-          }
-      }
-      __syncthreads();
-    }
-    if (tid < 16) {
-      float mm = fmaxf(fmaxf(m_s[0][tid], m_s[1][tid]), fmaxf(m_s[2][tid], m_s[3][tid]));
-      float ll = 0.f;
-      for (int w = 0; w < 4; w++) ll += m_s[w][tid] == -INFINITY ? 0.f : l_s[w][tid] * fast_exp2(m_s[w][tid] - mm);
-      pm[tid] = mm;
-      pl[tid] = ll;
-    }
-    for (int i = tid; i < 16 * D; i += 256) po[i] = o_s[i / D][i % D];
+    for (int kk = 0; kk < NK; kk++) kf[nt][kk] = ld16<v8>(kp + 32 * kk);
   }
+  f32x4 s[4];
+  float mw = -INFINITY;
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++) {
+    f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) c = E::mfma16(kf[nt][kk], qf[kk], c);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      c[r] = (k0 + 16 * nt + 4 * lg + r) < kend ? c[r] * p.qk_scale : -INFINITY;
+      mw = fmaxf(mw, c[r]);
+    }
+    s[nt] = c;
+  }
+  mw = column_max(mw);   // key k0 is visible, so the maximum is finite
+  float lw = 0.f;
+  v8 pf[2];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float x = fast_exp2(s[nt][r] - mw);
+      lw += x;
+      pf[nt >> 1][(nt & 1) * 4 + r] = (T)x;
+    }
+  lw = column_sum(lw);
+  // O^T[d][head] = V^T[d][key] P^T[key][head]; the transposing read hands lane (li, lg) column li of rows
+  // 4*lg..+3 of a 16-key tile
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  f32x4 acc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; dt++) {
+    acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      s16x4 x[2];
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const int row = 32 * c + 16 * u + 4 * lg + (li >> 2);
+        const int at = (row * CP + ((2 * dt + ((li >> 1) & 1) + 2 * row) & (CP - 1))) * 16 + (li & 1) * 8;
+        x[u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vs + at));
+      }
+      const s16x8 z = {x[0][0], x[0][1], x[0][2], x[0][3], x[1][0], x[1][1], x[1][2], x[1][3]};
+      acc[dt] = E::mfma16(__builtin_bit_cast(v8, z), pf[c], acc[dt]);
+    }
+  }
+  if (lg == 0) { pm[li] = mw; pl[li] = lw; }
+#pragma unroll
+  for (int dt = 0; dt < NDT; dt++) *reinterpret_cast<f32x4*>(po + li * D + 16 * dt + 4 * lg) = acc[dt];
+}
+
+// Sum / maximum over the 64 lanes of a wave, returned to every lane, in a fixed order.
+__device__ __forceinline__ float wave_sum_f32(float x) {
+  x += dpp_f32<0xB1>(x); x += dpp_f32<0x4E>(x); x += dpp_f32<0x141>(x); x += dpp_f32<0x140>(x);
+  return column_sum(x);
+}
+__device__ __forceinline__ float wave_max_f32(float x) {
+  x = fmaxf(x, dpp_f32<0xB1>(x)); x = fmaxf(x, dpp_f32<0x4E>(x)); x = fmaxf(x, dpp_f32<0x141>(x)); x = fmaxf(x, dpp_f32<0x140>(x));
+  return column_max(x);
 }
 
 // merge the chunk partials of one (sequence, query head); optionally keep the base-2 LSE.  The chunk maxima and
-// sums are read by different threads (independent loads, not a serial chain), the per-chunk weights go through LDS.
+// sums are read by different threads (independent loads, not a serial chain) and reduced inside each wave by
+// lane exchanges; two barriers per call instead of a barrier tree.  The per-chunk weights go through LDS.
 template <typename T, int D>
 __global__ void decode_merge_kernel(DecodeParams p, T* __restrict__ o, long long osb, long long osh, float* __restrict__ lse) {
   constexpr int WCAP = 256;  // chunk weights kept in LDS at a time
-  __shared__ float red[128];
+  __shared__ float red_m[2], red_l[2];
   __shared__ float w_s[WCAP];
-  const int hq_all = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
+  const int hq_all = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;   // nt = 64 or 128
+  const int wave = tid >> 6, nw = nt >> 6;
   const int h = hq_all / p.G, hq = hq_all % p.G, gt = hq / 16, col = hq % 16;
   const long long base = (((long long)b * p.Hkv + h) * p.GT + gt) * p.n_chunks;
   float m = -INFINITY;
   for (int c = tid; c < p.n_chunks; c += nt) m = fmaxf(m, p.pm[(base + c) * 16 + col]);
-  red[tid] = m;
+  m = wave_max_f32(m);
+  if ((tid & 63) == 0) red_m[wave] = m;
   __syncthreads();
-  for (int s = nt / 2; s > 0; s >>= 1) {
-    if (tid < s) red[tid] = fmaxf(red[tid], red[tid + s]);
-    __syncthreads();
-  }
-  m = red[0];
-  __syncthreads();
-  float l = 0.f;
-  for (int c = tid; c < p.n_chunks; c += nt) {
-    const float mc = p.pm[(base + c) * 16 + col];
-    if (mc != -INFINITY) l += p.pl[(base + c) * 16 + col] * fast_exp2(mc - m);
-  }
-  red[tid] = l;
-  __syncthreads();
-  for (int s = nt / 2; s > 0; s >>= 1) {
-    if (tid < s) red[tid] += red[tid + s];
-    __syncthreads();
-  }
-  l = red[0];
-  float acc = 0.f;  // this thread's output column d = tid (nt >= D is guaranteed by the launch)
+  m = nw == 2 ? fmaxf(red_m[0], red_m[1]) : red_m[0];
+  float l = 0.f, acc = 0.f;  // acc: this thread's output column d = tid (nt >= D is guaranteed by the launch)
   for (int c0 = 0; c0 < p.n_chunks; c0 += WCAP) {
     const int n = min(WCAP, p.n_chunks - c0);
-    __syncthreads();
+    if (c0 > 0) __syncthreads();   // the previous batch of weights has been used
     for (int c = tid; c < n; c += nt) {
       const float mc = p.pm[(base + c0 + c) * 16 + col];
-      w_s[c] = mc != -INFINITY ? fast_exp2(mc - m) : 0.f;
+      const float w = mc != -INFINITY ? fast_exp2(mc - m) : 0.f;
+      w_s[c] = w;
+      l += w * p.pl[(base + c0 + c) * 16 + col];
     }
     __syncthreads();
     if (tid < D) {
-#pragma unroll 4
+#pragma unroll 8
       for (int c = 0; c < n; c++) acc += p.po[((base + c0 + c) * 16 + col) * D + tid] * w_s[c];
     }
   }
+  l = wave_sum_f32(l);
+  if ((tid & 63) == 0) red_l[wave] = l;
+  __syncthreads();
+  l = nw == 2 ? red_l[0] + red_l[1] : red_l[0];
   if (tid < D) o[(long long)b * osb + (long long)hq_all * osh + tid] = (T)(l > 0.f ? acc / l : 0.f);
   if (lse && tid == 0) lse[(long long)b * p.Hkv * p.G + hq_all] = l > 0.f ? m + fast_log2(l) : INFINITY;
 }
@@ -192,48 +194,69 @@ struct ScoreParams {
 
 static constexpr int MAX_SCORE_BLOCKS = 8192;
 
+// One workgroup of SEL_NT threads per (kv-head, sequence): the work is a chain of short dependent phases, so
+// the aim is few round trips to memory and few barriers, not throughput.
+static constexpr int SEL_NT = 1024, SEL_NW = SEL_NT / 64;
+
 template <typename T, int D>
-__global__ __launch_bounds__(256) void decode_score_select_kernel(ScoreParams p) {
+__global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32;
   __shared__ float bscore[MAX_SCORE_BLOCKS];
   __shared__ int picked[64];
+  __shared__ long long wave_best[2][SEL_NW];
   const int h = blockIdx.x, b = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), li = lane & 15, lg = lane >> 4;
   const int lc = min(p.clens[b], p.slab_len);
   float* score = p.score + ((long long)b * p.Hkv + h) * p.slab_len;
-  // phase A: score[c] = sum over the group's heads of exp2(s*scale - lse)
-  for (int sub = wave; sub * 16 < lc; sub += 4) {
-    f32x4 tot = {0.f, 0.f, 0.f, 0.f};
-    const int key = sub * 16 + li;
-    const int row = key < lc ? key : 0;
-    const T* kp = (const T*)p.k + (long long)b * p.ksb + (long long)row * p.ksn + (long long)h * p.ksh + 8 * lg;
+  // phase A: score[c] = sum over the group's heads of exp2(s*scale - lse); a wave takes two 16-key tiles per
+  // trip and issues the K loads of both before it uses either
+  for (int sub0 = 2 * wave; sub0 * 16 < lc; sub0 += 2 * SEL_NW) {
+    v8 kf[2][NK];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int key = (sub0 + u) * 16 + li;
+      const int row = key < lc ? key : 0;
+      const T* kp = (const T*)p.k + (long long)b * p.ksb + (long long)row * p.ksn + (long long)h * p.ksh + 8 * lg;
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) kf[u][kk] = ld16<v8>(kp + 32 * kk);
+    }
+    f32x4 tot[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     for (int gt = 0; gt < p.GT; gt++) {
       const int hq = gt * 16 + li;
       const bool has_head = hq < p.G;
       const T* qp = (const T*)p.q + (long long)b * p.qsb + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
       const float l2 = has_head ? p.lse[(long long)b * p.Hkv * p.G + h * p.G + hq] : INFINITY;
-      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+      v8 qf[NK];
 #pragma unroll
-      for (int kk = 0; kk < NK; kk++) s = E::mfma16(ld16<v8>(kp + 32 * kk), has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>(), s);
+      for (int kk = 0; kk < NK; kk++) qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        float x = (sub * 16 + 4 * lg + r) < lc ? fast_exp2(s[r] * p.qk_scale - l2) : 0.f;
-        x += __shfl_xor(x, 1); x += __shfl_xor(x, 2); x += __shfl_xor(x, 4); x += __shfl_xor(x, 8);
-        tot[r] += x;
+      for (int u = 0; u < 2; u++) {
+        f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) sc = E::mfma16(kf[u][kk], qf[kk], sc);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          float x = ((sub0 + u) * 16 + 4 * lg + r) < lc ? fast_exp2(sc[r] * p.qk_scale - l2) : 0.f;
+          // sum over the 16 heads (the lanes of a row), in a fixed order
+          x += dpp_f32<0xB1>(x); x += dpp_f32<0x4E>(x); x += dpp_f32<0x141>(x); x += dpp_f32<0x140>(x);
+          tot[u][r] += x;
+        }
       }
     }
     if (li == 0) {
 #pragma unroll
-      for (int r = 0; r < 4; r++) if (sub * 16 + 4 * lg + r < lc) score[sub * 16 + 4 * lg + r] = tot[r];
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) if ((sub0 + u) * 16 + 4 * lg + r < lc) score[(sub0 + u) * 16 + 4 * lg + r] = tot[u][r];
     }
   }
   __syncthreads();
   // phase B: block scores
   const int a = p.ks / p.st, rr = p.bs / p.st, pad = a - 1;
   const int qb = (p.seqlens[b] - 1) / p.bs;
-  for (int blk = tid; blk < p.max_blocks; blk += 256) {
+  for (int blk = tid; blk < p.max_blocks; blk += SEL_NT) {
     float v = 0.f;
     if (blk < p.full_blocks) {
       for (int o = 0; o < a + rr - 1; o++) {
@@ -246,28 +269,25 @@ __global__ __launch_bounds__(256) void decode_score_select_kernel(ScoreParams p)
     if (blk < p.init_blocks || (blk <= qb && blk > qb - p.local_blocks)) v = INFINITY;
     bscore[blk] = v;
   }
-  __syncthreads();
-  // phase C: k_out rounds of (largest value, smallest index): wave-wide maxima of 64-bit (score, -index) keys,
-  // then the four wave results through LDS
-  __shared__ long long wave_best[4];
+  // phase C: k_out rounds of (largest value, smallest index).  A thread only ever reads the entries it wrote
+  // in phase B (blk = tid mod SEL_NT), and it is the owner that retires a winner, so no barrier is needed
+  // around bscore; the wave maxima alternate between two LDS rows, which leaves one barrier per round.
   for (int round = 0; round < p.k_out; round++) {
     float bv = -1.f;
     int bi = 0x7fffffff;
-    for (int blk = tid; blk < p.max_blocks; blk += 256) {
+    for (int blk = tid; blk < p.max_blocks; blk += SEL_NT) {
       const float v = bscore[blk];
       if (v > bv) { bv = v; bi = blk; }
     }
     const long long best = wave_max_i64(candidate_key(bv, bi));
-    if (lane == 0) wave_best[wave] = best;
+    if (lane == 0) wave_best[round & 1][wave] = best;
     __syncthreads();
-    if (tid == 0) {
-      long long m = wave_best[0];
-      for (int w = 1; w < 4; w++) m = wave_best[w] > m ? wave_best[w] : m;
-      const int win = candidate_index(m);
-      picked[round] = win;
-      bscore[win] = -2.f;
-    }
-    __syncthreads();
+    long long m = wave_best[round & 1][0];
+#pragma unroll
+    for (int w = 1; w < SEL_NW; w++) { const long long o = wave_best[round & 1][w]; m = o > m ? o : m; }
+    const int win = candidate_index(m);
+    if (tid == 0) picked[round] = win;
+    if ((win % SEL_NT) == tid) bscore[win] = -2.f;
   }
   // ascending order, ids beyond the query's block become -1 at the tail
   if (tid == 0) {
@@ -295,7 +315,7 @@ template <typename T, int D>
 static int run_decode(int mode, DecodeParams& p, void* o, long long osb, long long osh, float* lse, char* ws, hipStream_t s) {
   const size_t n = (size_t)p.B * p.Hkv * p.GT * p.n_chunks * 16;
   p.pm = (float*)ws; p.pl = p.pm + n; p.po = p.pl + n;
-  dim3 grid((unsigned)p.n_chunks, (unsigned)(p.Hkv * p.GT), (unsigned)p.B);
+  dim3 grid((unsigned)((p.n_chunks + 3) / 4), (unsigned)(p.Hkv * p.GT), (unsigned)p.B);
   if (mode == 0) decode_partial_kernel<T, D, 0><<<grid, 256, 0, s>>>(p);
   else decode_partial_kernel<T, D, 1><<<grid, 256, 0, s>>>(p);
   decode_merge_kernel<T, D><<<dim3((unsigned)(p.Hkv * p.G), (unsigned)p.B), D <= 64 ? 64 : 128, 0, s>>>(p, (T*)o, osb, osh, lse);
@@ -387,7 +407,7 @@ static int run_cmp_decode(DecodeParams& p, ScoreParams& sp, void* o, long long o
   if (rc != NSA_OK) return rc;
   if (sp.out_idx) {
     sp.lse = lse; sp.score = score;
-    decode_score_select_kernel<T, D><<<dim3((unsigned)p.Hkv, (unsigned)p.B), 256, 0, s>>>(sp);
+    decode_score_select_kernel<T, D><<<dim3((unsigned)p.Hkv, (unsigned)p.B), SEL_NT, 0, s>>>(sp);
   }
   return nsa_check_launch();
 }

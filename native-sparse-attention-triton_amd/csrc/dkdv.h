@@ -59,12 +59,6 @@ struct DkdvParams {
   float qk_scale, sm_scale;
 };
 
-// Asynchronous copies from global memory straight into LDS (no registers in between): every lane
-// supplies its own source address, the 64 lanes of a wave fill 64 consecutive 16-byte (4-byte) pieces
-// starting at the wave-uniform LDS address.  Completion is counted by vmcnt like any other load.
-typedef __attribute__((address_space(3))) void* nsa_lds_ptr;
-__device__ __forceinline__ void dma16(const void* src, unsigned char* lds) { __builtin_amdgcn_global_load_lds(src, (nsa_lds_ptr)lds, 16, 0, 0); }
-__device__ __forceinline__ void dma4(const void* src, unsigned char* lds) { __builtin_amdgcn_global_load_lds(src, (nsa_lds_ptr)lds, 4, 0, 0); }
 // Workgroup barrier that lets the n youngest vector-memory operations of each wave stay in flight: waits
 // for all LDS traffic and for all but n loads, then meets.  (__syncthreads() would wait for every
 // outstanding copy into LDS, including the ones meant to land during the next step.)

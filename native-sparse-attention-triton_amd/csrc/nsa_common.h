@@ -79,6 +79,12 @@ template <typename T> __device__ __forceinline__ float rounded(float x) {
 // of D + 8 elements halves the rate of the former and costs 40% on the latter.
 constexpr int lds_pitch(int d) { return d + 16; }
 
+// Asynchronous copies from global memory straight into LDS (no registers in between): every lane
+// supplies its own source address, the 64 lanes of a wave fill 64 consecutive 16-byte (4-byte) pieces
+// starting at the wave-uniform LDS address.  Completion is counted by vmcnt like any other load.
+typedef __attribute__((address_space(3))) void* nsa_lds_ptr;
+__device__ __forceinline__ void dma16(const void* src, unsigned char* lds) { __builtin_amdgcn_global_load_lds(src, (nsa_lds_ptr)lds, 16, 0, 0); }
+__device__ __forceinline__ void dma4(const void* src, unsigned char* lds) { __builtin_amdgcn_global_load_lds(src, (nsa_lds_ptr)lds, 4, 0, 0); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

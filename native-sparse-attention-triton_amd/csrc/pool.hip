@@ -25,7 +25,23 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(PoolParams p, T* __restri
   const T* wp = p.w ? (const T*)p.w + (long long)h * p.wsh : nullptr;
   const float wavg = 1.f / (float)p.ks;
   float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k = 0; k < p.ks; k++) {
+  // eight rows per trip, their loads issued together: a decode step pools a single window per sequence and is
+  // then bound by the round trips of this loop, not by bandwidth
+  int k = 0;
+  for (; k + 8 <= p.ks; k += 8) {
+    v8 xv[8];
+    float wk[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      xv[u] = ld16<v8>(xp + (long long)(k + u) * p.xsn);
+      wk[u] = wp ? (float)wp[k + u] : wavg;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc[j] += wk[u] * (float)xv[u][j];
+  }
+  for (; k < p.ks; k++) {
     const v8 xv = ld16<v8>(xp + (long long)k * p.xsn);
     const float wk = wp ? (float)wp[k] : wavg;
 #pragma unroll
