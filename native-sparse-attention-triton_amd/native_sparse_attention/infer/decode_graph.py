@@ -54,3 +54,10 @@ class NSADecodeGraph:
         self.gate.copy_(gate_value)
         self.graph.replay()
         return self.out
+
+    @torch.no_grad()
+    def replay(self) -> torch.Tensor:
+        """The same step for a caller that has already written the new token's states into `self.query`, `self.key`,
+        `self.value` and `self.gate` (for example as the `out=` of its projections): no copies, one graph launch."""
+        self.graph.replay()
+        return self.out

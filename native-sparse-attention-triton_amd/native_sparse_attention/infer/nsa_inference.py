@@ -35,8 +35,9 @@ def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, i
     batch = cu_seqlens.shape[0] - 1
     aux_cu = cache.staging_cu_seqlens(batch)
     stage = cache.before_compress_kv_cache[:, :batch].reshape(2, batch * kernel_size, cache.num_kv_heads, cache.head_dim)
-    key, _ = _compress_known_total(compress_func[0], batch, stage[0], weight[0], aux_cu, kernel_size, kernel_stride, intra_block_pe)
-    value, _ = _compress_known_total(compress_func[1], batch, stage[1], weight[1], aux_cu, kernel_size, kernel_stride)
+    out_cu = cache.staging_out_cu_seqlens(batch)
+    key, _ = _compress_known_total(compress_func[0], batch, out_cu, stage[0], weight[0], aux_cu, kernel_size, kernel_stride, intra_block_pe)
+    value, _ = _compress_known_total(compress_func[1], batch, out_cu, stage[1], weight[1], aux_cu, kernel_size, kernel_stride)
     if not need_cu:
         return key, value, None
     compress_cu_seqlens = torch.zeros(batch + 1, dtype=torch.int32, device=key.device)
@@ -44,11 +45,12 @@ def compress_infer(cu_seqlens, step, key, value, cache, weight, compress_func, i
     return key, value, compress_cu_seqlens
 
 
-def _compress_known_total(func, total, *args):
-    """Call a compression operator; this package's own operators are told the (host-known) number of output rows so
-    that they need not read it back from the device, any other callable gets the reference's arguments only."""
+def _compress_known_total(func, total, out_cu, *args):
+    """Call a compression operator; this package's own operators are told the (host-known) number of output rows and
+    their cu_seqlens so that they need neither read the one back from the device nor compute the other, any other
+    callable gets the reference's arguments only."""
     if func in (weightedpool_compress, avgpool_compress, linear_compress):
-        return func(*args, known_total=total)
+        return func(*args, known_total=total, known_y_cu=out_cu)
     return func(*args)
 
 

@@ -75,6 +75,7 @@ class NSACache:
         self.max_comp_length = (max_length - kernel_size) // kernel_stride + 1
         self.max_prompt_len = 0  # host copy of the longest prompt of the current batch (set at prefill)
         self._staging_cu = None
+        self._staging_out_cu = None
         self.static_shapes = False  # decode steps use the full slab extents instead of the current length bound
 
         def slab(rows):
@@ -99,6 +100,12 @@ class NSACache:
         if self._staging_cu is None:
             self._staging_cu = torch.arange(self.max_batch_size + 1, dtype=torch.int32, device=self.device) * self.kernel_size
         return self._staging_cu[: batch + 1]
+
+    def staging_out_cu_seqlens(self, batch: int) -> torch.Tensor:
+        """cu_seqlens of the compressed staging slab: one output row per sequence."""
+        if self._staging_out_cu is None:
+            self._staging_out_cu = torch.arange(self.max_batch_size + 1, dtype=torch.int32, device=self.device)
+        return self._staging_out_cu[: batch + 1]
 
     def max_seqlen(self, step: int) -> int:
         """Upper bound, known on the host, of every sequence's length at decode step `step`."""

@@ -42,7 +42,7 @@ def flash_attention_decode(q, k, v, seqlens, sm_scale: Optional[float] = None) -
     if sm_scale is None:
         sm_scale = 1 / math.sqrt(D)
     q, k, v = map(last_dim_contiguous, (q, k, v))
-    o = torch.zeros_like(q, memory_format=torch.contiguous_format)
+    o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     if L == 0:
         return o
     lib = _lib.load()
@@ -63,7 +63,7 @@ def topk_sparse_attention_decode(q, k, v, topk_idx, block_size: int, seqlens, sm
     if sm_scale is None:
         sm_scale = 1 / math.sqrt(D)
     q, k, v = map(last_dim_contiguous, (q, k, v))
-    o = torch.zeros_like(q, memory_format=torch.contiguous_format)
+    o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     if L == 0 or topk == 0:
         return o
     lib = _lib.load()
@@ -99,7 +99,7 @@ def compressed_attention_decode(
     if max_seqlen is None:
         max_seqlen = int(seqlens.max())  # fixes the output shape; the reference synchronises here too (:30)
     k_out = min(topk, math.ceil(max_seqlen / block_size))
-    o = torch.zeros_like(q, memory_format=torch.contiguous_format)
+    o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     idx = torch.empty(Hkv, B, k_out, dtype=torch.int32, device=q.device)
     lib = _lib.load()
     ws = _lib.workspace(lib.nsa_cmp_decode_workspace_bytes(B, Hq, Hkv, D, L), q.device)

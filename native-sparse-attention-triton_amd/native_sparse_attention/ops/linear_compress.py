@@ -10,7 +10,7 @@ from .utils import get_compressed_seqlens, last_dim_contiguous
 
 class LinearCompress(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w, cu_seqlens, kernel_size, kernel_stride, known_total=None):
+    def forward(ctx, x, w, cu_seqlens, kernel_size, kernel_stride, known_total=None, known_y_cu=None):
         assert x.dtype == torch.float16 or x.dtype == torch.bfloat16
         assert x.dtype == w.dtype
         assert cu_seqlens.dtype == torch.int32
@@ -24,7 +24,7 @@ class LinearCompress(torch.autograd.Function):
         assert head_dim % 8 == 0
         x = last_dim_contiguous(x)
         w = w.contiguous()
-        _, y_cu_seqlens = get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)
+        y_cu_seqlens = known_y_cu if known_y_cu is not None else get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)[1]
         # output shape: same host synchronisation as the reference (:366), unless the caller knows the total
         total_y = int(y_cu_seqlens[-1]) if known_total is None else int(known_total)
         y = torch.empty(total_y, num_heads, head_dim, dtype=x.dtype, device=x.device)
@@ -55,7 +55,7 @@ class LinearCompress(torch.autograd.Function):
             x.stride(0), x.stride(1), dy.stride(0), dy.stride(1), dx.stride(0), dx.stride(1),
             _lib.dtype_code(x), _lib.stream_ptr(x))
         _lib.check(rc, "nsa_linear_compress_bwd")
-        return dx, dw, None, None, None, None
+        return dx, dw, None, None, None, None, None
 
 
 def linear_compress(
@@ -66,6 +66,7 @@ def linear_compress(
     kernel_stride: int,
     pe: Optional[torch.Tensor] = None,
     known_total: Optional[int] = None,
+    known_y_cu: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Sliding-window linear projection of key/value states.
 
@@ -73,9 +74,10 @@ def linear_compress(
     [num_heads, kernel_size, head_dim], added as the bias pe[h].flatten() @ w[h].
     Returns (y [total_y, num_heads, head_dim], y_cu_seqlens int32).
     known_total (not in the reference's signature): total number of output rows when the caller knows it on the
-    host; the output is then allocated without reading y_cu_seqlens back.
+    host; the output is then allocated without reading y_cu_seqlens back.  known_y_cu (likewise): the output's
+    cu_seqlens when the caller already holds them.
     """
-    y, y_cu_seqlens = LinearCompress.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total)
+    y, y_cu_seqlens = LinearCompress.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu)
     if pe is not None:
         assert pe.dtype == x.dtype and pe.device == x.device
         bias = torch.einsum("hk,hkd->hd", pe.reshape(pe.shape[0], -1), w)

@@ -10,7 +10,7 @@ from .utils import get_compressed_seqlens, last_dim_contiguous
 
 class SlidingWindowWeightedPool(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w, cu_seqlens, kernel_size, kernel_stride, known_total=None):
+    def forward(ctx, x, w, cu_seqlens, kernel_size, kernel_stride, known_total=None, known_y_cu=None):
         assert x.dtype == torch.float16 or x.dtype == torch.bfloat16
         if w is not None:
             assert x.dtype == w.dtype
@@ -23,7 +23,7 @@ class SlidingWindowWeightedPool(torch.autograd.Function):
         assert kernel_size % kernel_stride == 0
         assert kernel_size in {16, 32, 64, 128}
         x = last_dim_contiguous(x)
-        y_seqlens, y_cu_seqlens = get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)
+        y_cu_seqlens = known_y_cu if known_y_cu is not None else get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)[1]
         # output shape: the one host synchronisation the reference has too, unless the caller knows the total
         total_y = int(y_cu_seqlens[-1]) if known_total is None else int(known_total)
         y = torch.empty(total_y, num_heads, head_dim, dtype=x.dtype, device=x.device)
@@ -57,7 +57,7 @@ class SlidingWindowWeightedPool(torch.autograd.Function):
             w.stride(0) if w is not None else 0, dw.stride(0) if w is not None else 0,
             _lib.dtype_code(x), ws.data_ptr(), ws.numel(), _lib.stream_ptr(x))
         _lib.check(rc, "nsa_pool_bwd")
-        return dx, dw, None, None, None, None
+        return dx, dw, None, None, None, None, None
 
 
 def weightedpool_compress(
@@ -68,6 +68,7 @@ def weightedpool_compress(
     kernel_stride: int,
     pe: Optional[torch.Tensor] = None,
     known_total: Optional[int] = None,
+    known_y_cu: Optional[torch.Tensor] = None,
 ):
     """Weighted sliding-window pooling of key/value states.
 
@@ -75,9 +76,10 @@ def weightedpool_compress(
     [num_heads, kernel_size, head_dim] intra-block positional embedding, added as the bias
     sum_k w[h,k] pe[h,k,:].  Returns (y [total_y, num_heads, head_dim], y_cu_seqlens int32).
     known_total (not in the reference's signature): total number of output rows when the caller knows it on the
-    host; the output is then allocated without reading y_cu_seqlens back.
+    host; the output is then allocated without reading y_cu_seqlens back.  known_y_cu (likewise): the output's
+    cu_seqlens when the caller already holds them (a decode step compresses one full window per sequence).
     """
-    y, y_cu_seqlens = SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total)
+    y, y_cu_seqlens = SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu)
     if pe is not None:
         assert pe.dtype == x.dtype and pe.device == x.device
         bias = torch.einsum("hkd,hk->hd", pe, w)
@@ -93,10 +95,12 @@ def avgpool_compress(
     kernel_stride: int,
     pe: Optional[torch.Tensor] = None,
     known_total: Optional[int] = None,
+    known_y_cu: Optional[torch.Tensor] = None,
 ):
-    """Average sliding-window pooling; ``w`` must be None.  Bias = mean_k pe[h,k,:].  known_total as in weightedpool_compress."""
+    """Average sliding-window pooling; ``w`` must be None.  Bias = mean_k pe[h,k,:].  known_total / known_y_cu as in
+    weightedpool_compress."""
     assert w is None, "don't need additional weight for avgpool"
-    y, y_cu_seqlens = SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total)
+    y, y_cu_seqlens = SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu)
     if pe is not None:
         assert pe.dtype == x.dtype and pe.device == x.device
         y = y + torch.mean(pe, dim=1).unsqueeze(0)
