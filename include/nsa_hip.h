@@ -255,6 +255,24 @@ int nsa_cache_commit_token(const void* const* tokens, const int64_t* strides, co
                            int64_t batch, int64_t num_kv_heads, int64_t head_dim, int64_t max_batch, int64_t kernel_size,
                            int64_t compress_rows, int64_t sparse_rows, int64_t window_size, void* stream);
 
+/* One decode step's work ahead of its attention branches in a single launch, for caches whose compression is
+ * a (weighted) average pool: nsa_cache_stage_token, the pooling of a completed window
+ * (ops/triton/weighted_pool.py:182-279 on the staging slab, as compress_infer of infer/inference_func.py:27-75
+ * calls it), the three rotations of infer/nsa_inference.py:96-112 with positions sparse_len[b] (query, key) and
+ * compress_len[b] * kernel_stride (compressed key), and nsa_cache_commit_token.  q [batch,Hq,D], k, v
+ * [batch,Hkv,D]; q_out receives the rotated query.  pool_weight_k / pool_weight_v: contiguous [Hkv,kernel_size]
+ * or NULL for the plain average; bias_k: optional contiguous [Hkv,D] added to the pooled key (the intra-block
+ * position term).  strides: HOST int64[8] = q(b,h) k(b,h) v(b,h) q_out(b,h).  Cache contents, lengths and the
+ * rotated query equal those of the separate entry points bit for bit.
+ */
+int nsa_decode_prepare(const void* q, const void* k, const void* v, void* q_out, const void* pool_weight_k,
+                       const void* pool_weight_v, const void* bias_k, const float* inv_freq, float attention_scaling,
+                       void* stage_slab, int32_t* stage_len, void* compress_slab, int32_t* compress_len, void* sparse_slab,
+                       int32_t* sparse_len, void* sliding_slab, int32_t* sliding_len, int64_t batch, int64_t num_q_heads,
+                       int64_t num_kv_heads, int64_t head_dim, const int64_t* strides, int64_t max_batch, int64_t kernel_size,
+                       int64_t kernel_stride, int64_t compress_rows, int64_t sparse_rows, int64_t window_size, int dtype,
+                       void* stream);
+
 /* ---- gated sum of the three branches -----------------------------------------------------------
  * out[n, h, :] = gate[n, h, 0] * branch0 + gate[n, h, 1] * branch1 + gate[n, h, 2] * branch2, rounded step by
  * step like the tensor expression of native_sparse_attention/infer/nsa_inference.py:146-150.

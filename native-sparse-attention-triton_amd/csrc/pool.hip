@@ -39,13 +39,13 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(PoolParams p, T* __restri
 #pragma unroll
     for (int u = 0; u < 8; u++)
 #pragma unroll
-      for (int j = 0; j < 8; j++) acc[j] += wk[u] * (float)xv[u][j];
+      for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(wk[u], (float)xv[u][j], acc[j]);
   }
   for (; k < p.ks; k++) {
     const v8 xv = ld16<v8>(xp + (long long)k * p.xsn);
     const float wk = wp ? (float)wp[k] : wavg;
 #pragma unroll
-    for (int j = 0; j < 8; j++) acc[j] += wk * (float)xv[j];
+    for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(wk, (float)xv[j], acc[j]);
   }
   v8 out;
 #pragma unroll

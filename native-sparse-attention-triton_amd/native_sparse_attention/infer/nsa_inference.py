@@ -130,6 +130,15 @@ def nsa_infer(
     """Gated sum of the compressed, selected and sliding-window branches; same shape as ``query``."""
     if step == 0:
         cache.reset()
+    if step > 0 and _single_launch_prepare_applies(rope, cache, compress_func):
+        # pooling compression and this package's rotary module: everything up to the attention branches is one kernel
+        assert cache.static_shapes or cache.max_seqlen(step) <= cache.max_length, "cache slab too short for this decode step"
+        with torch.no_grad():
+            wk, wv = (None if w is None else w.detach().contiguous() for w in compress_weight)
+            query = cache.decode_prepare(query, key, value, rope._frequencies(), rope.attention_scaling, wk, wv,
+                                         _pooled_position_bias(compress_func[0], wk, intra_block_pe))
+        return _decode_branches(cu_seqlens, step, query, key, value, gate_value, cache, kernel_size, kernel_stride, block_size, topk,
+                                init_blocks, local_blocks, window_size, return_branches)
     cache.prepare_compress(cu_seqlens, step, key, value)
     # In a decode step every position is a cache length that lives on the device: this package's rotary module can
     # take them from there, any other rope callable gets the reference's (cu_seqlens, step) arguments.
@@ -149,6 +158,34 @@ def nsa_infer(
     cache.update_kv(cu_seqlens, step, compress_key, compress_value, key, value, key, value)
     cmp_out, topk_idx = compressed_attention_infer(cu_seqlens, step, query, compress_key, compress_value, cache, kernel_size,
                                                    kernel_stride, topk, block_size, init_blocks, local_blocks)
+    sparse_out = topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size)
+    window_out = sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size)
+    out = gate_combine(gate_value, cmp_out, sparse_out, window_out)
+    if return_branches:
+        return out, (cmp_out, sparse_out, window_out, topk_idx)
+    return out
+
+
+def _single_launch_prepare_applies(rope, cache, compress_func) -> bool:
+    return (hasattr(rope, "rotate_at") and hasattr(rope, "_frequencies") and hasattr(cache, "decode_prepare")
+            and all(f in (weightedpool_compress, avgpool_compress) for f in compress_func) and compress_func[0] is compress_func[1])
+
+
+def _pooled_position_bias(func, weight, intra_block_pe):
+    """The term the pooling operators add to a compressed key for the intra-block position embedding
+    (weighted_pool.py:318-321 and :360-362 of the reference), as they compute it."""
+    if intra_block_pe is None:
+        return None
+    if func is weightedpool_compress:
+        return torch.einsum("hkd,hk->hd", intra_block_pe, weight).contiguous()
+    return torch.mean(intra_block_pe, dim=1).contiguous()
+
+
+def _decode_branches(cu_seqlens, step, query, key, value, gate_value, cache, kernel_size, kernel_stride, block_size, topk, init_blocks,
+                     local_blocks, window_size, return_branches):
+    """The three attention branches of a decode step over the updated cache, and their gated sum."""
+    cmp_out, topk_idx = compressed_attention_infer(cu_seqlens, step, query, None, None, cache, kernel_size, kernel_stride, topk,
+                                                   block_size, init_blocks, local_blocks)
     sparse_out = topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size)
     window_out = sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size)
     out = gate_combine(gate_value, cmp_out, sparse_out, window_out)

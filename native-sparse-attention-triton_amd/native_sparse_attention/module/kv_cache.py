@@ -140,6 +140,35 @@ class NSACache:
                                                    self.max_batch_size, self.kernel_size, self.kernel_stride, _lib.stream_ptr(key))
             _lib.check(rc, "nsa_cache_stage_token")
 
+    # ---- a whole decode step's cache work in one launch ---------------------------------------
+    @torch.no_grad()
+    def decode_prepare(self, query, key, value, inv_freq, attention_scaling, weight_k=None, weight_v=None, bias_k=None):
+        """prepare_compress + pooling of a completed window + rotary embedding of query, key and compressed key +
+        update_kv for one new token per sequence, as a single kernel (pooling compression only: weight_k / weight_v
+        [num_kv_heads, kernel_size] or None for the plain average, bias_k [num_kv_heads, head_dim] the optional
+        position term of the pooled key).  Returns the rotated query.  Same cache contents as the separate calls."""
+        batch = query.shape[0]
+        assert batch <= self.max_batch_size and key.shape == value.shape == (batch, self.num_kv_heads, self.head_dim)
+        assert query.shape[2] == self.head_dim and query.dtype == key.dtype == value.dtype == self.dtype
+        assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and inv_freq.shape[0] == self.head_dim // 2
+        query, key, value = last_dim_contiguous(query), last_dim_contiguous(key), last_dim_contiguous(value)
+        for w in (weight_k, weight_v):
+            assert w is None or (w.dtype == self.dtype and w.is_contiguous() and w.shape == (self.num_kv_heads, self.kernel_size))
+        assert bias_k is None or (bias_k.dtype == self.dtype and bias_k.is_contiguous() and bias_k.shape == (self.num_kv_heads, self.head_dim))
+        out = torch.empty_like(query, memory_format=torch.contiguous_format)
+        strides = _lib.host_i64([query.stride(0), query.stride(1), key.stride(0), key.stride(1), value.stride(0), value.stride(1),
+                                 out.stride(0), out.stride(1)])
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        rc = _lib.load().nsa_decode_prepare(
+            query.data_ptr(), key.data_ptr(), value.data_ptr(), out.data_ptr(), ptr(weight_k), ptr(weight_v), ptr(bias_k),
+            inv_freq.data_ptr(), float(attention_scaling), self.before_compress_kv_cache.data_ptr(), self.before_compress_kv_len.data_ptr(),
+            self.compress_kv_cache.data_ptr(), self.compress_kv_len.data_ptr(), self.sparse_kv_cache.data_ptr(),
+            self.sparse_kv_len.data_ptr(), self.sliding_kv_cache.data_ptr(), self.sliding_kv_len.data_ptr(), batch, query.shape[1],
+            self.num_kv_heads, self.head_dim, strides, self.max_batch_size, self.kernel_size, self.kernel_stride, self.max_comp_length,
+            self.max_length, self.window_size, _lib.dtype_code(query), _lib.stream_ptr(query))
+        _lib.check(rc, "nsa_decode_prepare")
+        return out
+
     # ---- after rope ---------------------------------------------------------------------------
     def update_kv(self, cu_seqlens, step, compress_key, compress_value, sparse_key, sparse_value, sliding_key, sliding_value):
         assert compress_key.shape == compress_value.shape and sparse_key.shape == sparse_value.shape

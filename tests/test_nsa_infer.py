@@ -156,3 +156,52 @@ def test_graphed_decode_step_equals_eager_steps(device):
             assert torch.equal(getattr(caches[0], name), getattr(caches[1], name)), (name, step)
     n = int(caches[1].sparse_kv_len[2])
     assert torch.equal(caches[0].sparse_kv_cache[:, 2, :n], caches[1].sparse_kv_cache[:, 2, :n])
+
+
+@pytest.mark.parametrize("weighted,with_pe,dtype", [(True, True, torch.bfloat16), (True, False, torch.float16), (False, True, torch.bfloat16)])
+def test_single_launch_prepare_equals_separate_operators(device, weighted, with_pe, dtype):
+    """The decode step whose cache work is one kernel (pooling compression + this package's rotary module) against the
+    same step built from the separate operators (forced by handing the compression in as plain callables), on two
+    identically prefilled caches: outputs, lengths and every valid cache row must be identical, window completions,
+    staging shifts and ring wrap-around included."""
+    from native_sparse_attention.module import RopeConfig, RotaryEmbedding
+    from native_sparse_attention.ops import avgpool_compress
+    Hq, Hkv, d, ks, st, bs, topk, W = 16, 2, 128, 32, 16, 64, 4, 64
+    lens, steps = [300, 47, 20, 1100], 70
+    B = len(lens)
+    g = torch.Generator(device=device).manual_seed(11)
+    cu = cu_from_lens(lens, device)
+    T = int(cu[-1])
+    rope = RotaryEmbedding(RopeConfig(head_dim=d), device=device)
+
+    def rnd(*shape):
+        return torch.randn(*shape, generator=g, device=device).to(dtype)
+
+    if weighted:
+        weights = (torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).to(dtype),
+                   torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).to(dtype))
+        fn = weightedpool_compress
+    else:
+        weights, fn = (None, None), avgpool_compress
+    pe = (rnd(Hkv, ks, d).float() * 0.02).to(dtype) if with_pe else None
+    plain = lambda *a, **kw: fn(*a, **kw)   # not recognised as a pooling operator: the separate-operator path runs
+    q0, k0, v0, g0 = rnd(T, Hq, d), rnd(T, Hkv, d), rnd(T, Hkv, d), torch.sigmoid(rnd(T, Hq, 3).float()).to(dtype)
+    caches = [NSACache(B, max(lens) + steps + 8, Hkv, d, ks, st, W, dtype, device) for _ in range(2)]
+    tails = [(weights, (fn, fn), pe, ks, st, bs, topk, 1, 2, W), (weights, (plain, plain), pe, ks, st, bs, topk, 1, 2, W)]
+    for c, tail in zip(caches, tails):
+        nsa_infer(cu, 0, q0, k0, v0, g0, rope, c, *tail)
+    for step in range(1, steps + 1):
+        kv = rnd(B, Hkv + 1, 2 * d)
+        q, k, v, gt = rnd(B, Hq, d), kv[:, :Hkv, :d], kv[:, 1:, d:], torch.sigmoid(rnd(B, Hq, 3).float()).to(dtype)   # strided k, v
+        got = nsa_infer(cu, step, q, k, v, gt, rope, caches[0], *tails[0])
+        want = nsa_infer(cu, step, q, k, v, gt, rope, caches[1], *tails[1])
+        assert torch.equal(got, want), step
+        for name in ("sparse_kv_len", "compress_kv_len", "before_compress_kv_len", "sliding_kv_len"):
+            assert torch.equal(getattr(caches[0], name), getattr(caches[1], name)), (name, step)
+    for b in range(B):
+        for slab, ln in (("sparse_kv_cache", "sparse_kv_len"), ("compress_kv_cache", "compress_kv_len"),
+                         ("before_compress_kv_cache", "before_compress_kv_len")):
+            n = int(getattr(caches[1], ln)[b])
+            assert torch.equal(getattr(caches[0], slab)[:, b, :n], getattr(caches[1], slab)[:, b, :n]), (slab, b)
+        n = min(int(caches[1].sliding_kv_len[b]), W)
+        assert torch.equal(caches[0].sliding_kv_cache[:, b, :n], caches[1].sliding_kv_cache[:, b, :n]), ("ring", b)
