@@ -196,7 +196,7 @@ static constexpr int MAX_SCORE_BLOCKS = 8192;
 
 // One workgroup of SEL_NT threads per (kv-head, sequence): the work is a chain of short dependent phases, so
 // the aim is few round trips to memory and few barriers, not throughput.
-static constexpr int SEL_NT = 1024, SEL_NW = SEL_NT / 64;
+static constexpr int SEL_NT = 1024, SEL_NW = SEL_NT / 64, SEL_LDS_SCORES = 8192;
 
 template <typename T, int D>
 __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams p) {
@@ -209,7 +209,10 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
   const int h = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), li = lane & 15, lg = lane >> 4;
   const int lc = min(p.clens[b], p.slab_len);
-  float* score = p.score + ((long long)b * p.Hkv + h) * p.slab_len;
+  const int qb = (p.seqlens[b] - 1) / p.bs;
+  // per-key scores stay in LDS when they fit (a round trip to memory less), else in the workspace
+  __shared__ float score_s[SEL_LDS_SCORES];
+  float* score = lc <= SEL_LDS_SCORES ? score_s : p.score + ((long long)b * p.Hkv + h) * p.slab_len;
   // phase A: score[c] = sum over the group's heads of exp2(s*scale - lse); a wave takes two 16-key tiles per
   // trip and issues the K loads of both before it uses either
   for (int sub0 = 2 * wave; sub0 * 16 < lc; sub0 += 2 * SEL_NW) {
@@ -255,7 +258,6 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
   __syncthreads();
   // phase B: block scores
   const int a = p.ks / p.st, rr = p.bs / p.st, pad = a - 1;
-  const int qb = (p.seqlens[b] - 1) / p.bs;
   for (int blk = tid; blk < p.max_blocks; blk += SEL_NT) {
     float v = 0.f;
     if (blk < p.full_blocks) {
@@ -271,7 +273,11 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
   }
   // phase C: k_out rounds of (largest value, smallest index).  A thread only ever reads the entries it wrote
   // in phase B (blk = tid mod SEL_NT), and it is the owner that retires a winner, so no barrier is needed
-  // around bscore; the wave maxima alternate between two LDS rows, which leaves one barrier per round.
+  // around bscore; the wave maxima alternate between two LDS rows, which leaves one barrier per round.  Waves
+  // that own no block leave first (a barrier only counts the waves that are still alive), so with up to 64
+  // blocks a round is a single wave's lane exchanges.
+  const int nwc = min(SEL_NW, (p.max_blocks + 63) / 64);
+  if (wave >= nwc) return;
   for (int round = 0; round < p.k_out; round++) {
     float bv = -1.f;
     int bi = 0x7fffffff;
@@ -279,12 +285,13 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
       const float v = bscore[blk];
       if (v > bv) { bv = v; bi = blk; }
     }
-    const long long best = wave_max_i64(candidate_key(bv, bi));
-    if (lane == 0) wave_best[round & 1][wave] = best;
-    __syncthreads();
-    long long m = wave_best[round & 1][0];
-#pragma unroll
-    for (int w = 1; w < SEL_NW; w++) { const long long o = wave_best[round & 1][w]; m = o > m ? o : m; }
+    long long m = wave_max_i64(candidate_key(bv, bi));
+    if (nwc > 1) {
+      if (lane == 0) wave_best[round & 1][wave] = m;
+      __syncthreads();
+      m = wave_best[round & 1][0];
+      for (int w = 1; w < nwc; w++) { const long long o = wave_best[round & 1][w]; m = o > m ? o : m; }
+    }
     const int win = candidate_index(m);
     if (tid == 0) picked[round] = win;
     if ((win % SEL_NT) == tid) bscore[win] = -2.f;
