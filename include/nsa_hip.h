@@ -273,6 +273,25 @@ int nsa_decode_prepare(const void* q, const void* k, const void* v, void* q_out,
                        int64_t kernel_stride, int64_t compress_rows, int64_t sparse_rows, int64_t window_size, int dtype,
                        void* stream);
 
+/* The selected-block branch, the sliding-window branch and the gated sum of a decode step in two launches
+ * (one for the partials of both branches, one for both merges and the gate) instead of five: the calls of
+ * topk_sparse_attention_infer and sliding_window_attention_infer (infer/inference_func.py:140-202) and the gate
+ * expression of infer/nsa_inference.py:146-150.  Arguments as for nsa_topk_decode / nsa_dense_decode /
+ * nsa_gate_combine; cmp_out is the compressed branch's output [batch,Hq,D]; o_topk / o_window receive the two
+ * branch outputs, out the gated sum.  strides: HOST int64[28] =
+ *   q(b,h) sparse_k(b,n,h) sparse_v(b,n,h) idx(h,b,k) window_k(b,n,h) window_v(b,n,h) cmp_out(b,h) gate(b,h,k)
+ *   out(b,h) o_topk(b,h) o_window(b,h).
+ * Every result equals that of the separate entry points bit for bit.
+ */
+size_t nsa_decode_branches_gate_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                                int64_t window_rows, int64_t topk, int64_t block_size);
+int nsa_decode_branches_gate(const void* q, const void* sparse_k, const void* sparse_v, const int32_t* sparse_len,
+                             const int32_t* topk_idx, const void* window_k, const void* window_v, const int32_t* window_len,
+                             const void* cmp_out, const void* gate, void* out, void* o_topk, void* o_window, int64_t batch,
+                             int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t sparse_rows,
+                             int64_t window_rows, int64_t topk, int64_t block_size, const int64_t* strides, float sm_scale,
+                             int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- gated sum of the three branches -----------------------------------------------------------
  * out[n, h, :] = gate[n, h, 0] * branch0 + gate[n, h, 1] * branch1 + gate[n, h, 2] * branch2, rounded step by
  * step like the tensor expression of native_sparse_attention/infer/nsa_inference.py:146-150.

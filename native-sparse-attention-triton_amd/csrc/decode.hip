@@ -22,16 +22,20 @@ struct DecodeParams {
 // of the chunk are copied straight from global memory into a wave-private LDS tile (no registers, no
 // ds_write) while the scores are formed; rows are 256 bytes, unpadded, with the 16-byte pieces of row r
 // rotated by 2r positions so that the transposing reads hit every bank once.
+template <int D> struct DecodeTile {
+  static constexpr int CP = D > 64 ? 16 : (D > 32 ? 8 : 4);   // 16-byte pieces per staged row
+  static constexpr int BYTES = 64 * CP * 16;                  // one wave's V tile
+};
+
 template <typename T, int D, int MODE>
-__global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
+__device__ __forceinline__ void decode_partial_body(const DecodeParams& p, int block_x, unsigned char* vs_all) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32, NDT = D / 16;
-  constexpr int CP = D > 64 ? 16 : (D > 32 ? 8 : 4);   // 16-byte pieces per staged row
+  constexpr int CP = DecodeTile<D>::CP;
   constexpr int RPI = 64 / CP;                         // rows per 1 KiB wave-copy
-  __shared__ __attribute__((aligned(256))) unsigned char v_s[4][64 * CP * 16];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, lg = lane >> 4;
-  const int chunk = blockIdx.x * 4 + wave, h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT, b = blockIdx.z;
+  const int chunk = block_x * 4 + wave, h = blockIdx.y / p.GT, gt = blockIdx.y % p.GT, b = blockIdx.z;
   if (chunk >= p.n_chunks) return;
   const int len = min(p.lens[b], p.slab_len);  // never read past the slab
   int k0, kend;  // keys [k0, kend) of this chunk are visible
@@ -57,7 +61,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
   }
   // V rows -> LDS, started first.  Rows past kend are copied from row k0 (slab rows past the length may hold
   // anything, and 0 * NaN would poison the sum); their probabilities are exactly 0.
-  unsigned char* vs = v_s[wave];
+  unsigned char* vs = vs_all + wave * DecodeTile<D>::BYTES;
 #pragma unroll
   for (int i = 0; i < 64 / RPI; i++) {
     const int row = i * RPI + lane / CP;
@@ -131,6 +135,20 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
   for (int dt = 0; dt < NDT; dt++) *reinterpret_cast<f32x4*>(po + li * D + 16 * dt + 4 * lg) = acc[dt];
 }
 
+template <typename T, int D, int MODE>
+__global__ __launch_bounds__(256) void decode_partial_kernel(DecodeParams p) {
+  __shared__ __attribute__((aligned(256))) unsigned char v_s[4 * DecodeTile<D>::BYTES];
+  decode_partial_body<T, D, MODE>(p, blockIdx.x, v_s);
+}
+
+// the partials of the selected-block branch (first blocks_a workgroups in x) and of a dense branch in one launch
+template <typename T, int D>
+__global__ __launch_bounds__(256) void decode_partial_pair_kernel(DecodeParams pa, DecodeParams pb, int blocks_a) {
+  __shared__ __attribute__((aligned(256))) unsigned char v_s[4 * DecodeTile<D>::BYTES];
+  if ((int)blockIdx.x < blocks_a) decode_partial_body<T, D, 1>(pa, blockIdx.x, v_s);
+  else decode_partial_body<T, D, 0>(pb, blockIdx.x - blocks_a, v_s);
+}
+
 // Sum / maximum over the 64 lanes of a wave, returned to every lane, in a fixed order.
 __device__ __forceinline__ float wave_sum_f32(float x) {
   x += dpp_f32<0xB1>(x); x += dpp_f32<0x4E>(x); x += dpp_f32<0x141>(x); x += dpp_f32<0x140>(x);
@@ -141,24 +159,22 @@ __device__ __forceinline__ float wave_max_f32(float x) {
   return column_max(x);
 }
 
-// merge the chunk partials of one (sequence, query head); optionally keep the base-2 LSE.  The chunk maxima and
-// sums are read by different threads (independent loads, not a serial chain) and reduced inside each wave by
-// lane exchanges; two barriers per call instead of a barrier tree.  The per-chunk weights go through LDS.
-template <typename T, int D>
-__global__ void decode_merge_kernel(DecodeParams p, T* __restrict__ o, long long osb, long long osh, float* __restrict__ lse) {
+struct MergeScratch { float red_m[2], red_l[2]; float w_s[256]; };
+
+// Merged output column d = tid of one (sequence, query head): sum_c w_c O_c[d] / sum_c w_c l_c; m_out / l_out
+// receive the maximum and the sum.  Called by all threads of the workgroup (blockDim = 64 or 128).
+template <int D>
+__device__ __forceinline__ float decode_merge_body(const DecodeParams& p, int hq_all, int b, MergeScratch& sh, float& m_out, float& l_out) {
   constexpr int WCAP = 256;  // chunk weights kept in LDS at a time
-  __shared__ float red_m[2], red_l[2];
-  __shared__ float w_s[WCAP];
-  const int hq_all = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;   // nt = 64 or 128
-  const int wave = tid >> 6, nw = nt >> 6;
+  const int tid = threadIdx.x, nt = blockDim.x, wave = tid >> 6, nw = nt >> 6;
   const int h = hq_all / p.G, hq = hq_all % p.G, gt = hq / 16, col = hq % 16;
   const long long base = (((long long)b * p.Hkv + h) * p.GT + gt) * p.n_chunks;
   float m = -INFINITY;
   for (int c = tid; c < p.n_chunks; c += nt) m = fmaxf(m, p.pm[(base + c) * 16 + col]);
   m = wave_max_f32(m);
-  if ((tid & 63) == 0) red_m[wave] = m;
+  if ((tid & 63) == 0) sh.red_m[wave] = m;
   __syncthreads();
-  m = nw == 2 ? fmaxf(red_m[0], red_m[1]) : red_m[0];
+  m = nw == 2 ? fmaxf(sh.red_m[0], sh.red_m[1]) : sh.red_m[0];
   float l = 0.f, acc = 0.f;  // acc: this thread's output column d = tid (nt >= D is guaranteed by the launch)
   for (int c0 = 0; c0 < p.n_chunks; c0 += WCAP) {
     const int n = min(WCAP, p.n_chunks - c0);
@@ -166,21 +182,61 @@ __global__ void decode_merge_kernel(DecodeParams p, T* __restrict__ o, long long
     for (int c = tid; c < n; c += nt) {
       const float mc = p.pm[(base + c0 + c) * 16 + col];
       const float w = mc != -INFINITY ? fast_exp2(mc - m) : 0.f;
-      w_s[c] = w;
+      sh.w_s[c] = w;
       l += w * p.pl[(base + c0 + c) * 16 + col];
     }
     __syncthreads();
     if (tid < D) {
 #pragma unroll 8
-      for (int c = 0; c < n; c++) acc += p.po[((base + c0 + c) * 16 + col) * D + tid] * w_s[c];
+      for (int c = 0; c < n; c++) acc += p.po[((base + c0 + c) * 16 + col) * D + tid] * sh.w_s[c];
     }
   }
   l = wave_sum_f32(l);
-  if ((tid & 63) == 0) red_l[wave] = l;
+  if ((tid & 63) == 0) sh.red_l[wave] = l;
   __syncthreads();
-  l = nw == 2 ? red_l[0] + red_l[1] : red_l[0];
-  if (tid < D) o[(long long)b * osb + (long long)hq_all * osh + tid] = (T)(l > 0.f ? acc / l : 0.f);
+  l = nw == 2 ? sh.red_l[0] + sh.red_l[1] : sh.red_l[0];
+  m_out = m; l_out = l;
+  return l > 0.f ? acc / l : 0.f;
+}
+
+// merge the chunk partials of one (sequence, query head); optionally keep the base-2 LSE.  The chunk maxima and
+// sums are read by different threads (independent loads, not a serial chain) and reduced inside each wave by
+// lane exchanges; two barriers per call instead of a barrier tree.  The per-chunk weights go through LDS.
+template <typename T, int D>
+__global__ void decode_merge_kernel(DecodeParams p, T* __restrict__ o, long long osb, long long osh, float* __restrict__ lse) {
+  __shared__ MergeScratch sh;
+  const int hq_all = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  float m, l;
+  const float val = decode_merge_body<D>(p, hq_all, b, sh, m, l);
+  if (tid < D) o[(long long)b * osb + (long long)hq_all * osh + tid] = (T)val;
   if (lse && tid == 0) lse[(long long)b * p.Hkv * p.G + hq_all] = l > 0.f ? m + fast_log2(l) : INFINITY;
+}
+
+// Merges of the selected-block branch (pa) and of the sliding-window branch (pb), and the gated sum with the
+// compressed branch, out = g0 * cmp + g1 * sel + g2 * win, every product and partial sum rounded to the element
+// type in that order (the arithmetic of the tensor expression); the two branch outputs are stored as well.
+struct GateParams {
+  const void* cmp; const void* gate; void* out; void* o_a; void* o_b;
+  long long csb, csh, gsb, gsh, gsk, osb, osh, asb, ash, bsb, bsh;
+};
+template <typename T, int D>
+__global__ void decode_merge_pair_gate_kernel(DecodeParams pa, DecodeParams pb, GateParams g) {
+  __shared__ MergeScratch sh;
+  const int hq_all = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  float m, l;
+  const float va = decode_merge_body<D>(pa, hq_all, b, sh, m, l);
+  __syncthreads();   // the scratch is reused
+  const float vb = decode_merge_body<D>(pb, hq_all, b, sh, m, l);
+  if (tid < D) {
+    const T ta = (T)va, tb = (T)vb;
+    ((T*)g.o_a)[(long long)b * g.asb + (long long)hq_all * g.ash + tid] = ta;
+    ((T*)g.o_b)[(long long)b * g.bsb + (long long)hq_all * g.bsh + tid] = tb;
+    const T* gp = (const T*)g.gate + (long long)b * g.gsb + (long long)hq_all * g.gsh;
+    const float g0 = (float)gp[0], g1 = (float)gp[g.gsk], g2 = (float)gp[2 * g.gsk];
+    const float c = (float)((const T*)g.cmp)[(long long)b * g.csb + (long long)hq_all * g.csh + tid];
+    const float x = rounded<T>(g0 * c), y = rounded<T>(g1 * (float)ta), z = rounded<T>(g2 * (float)tb);
+    ((T*)g.out)[(long long)b * g.osb + (long long)hq_all * g.osh + tid] = (T)(rounded<T>(x + y) + z);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -445,6 +501,59 @@ extern "C" int nsa_cmp_decode(const void* q, const void* k, const void* v, const
   const size_t part = cmp_decode_partial(batch, num_q_heads, num_kv_heads, head_dim, slab_len);
   hipStream_t s = (hipStream_t)stream;
 #define CALL(T, D) run_cmp_decode<T, D>(p, sp, o, osb, osh, (char*)workspace, part, s)
+  DECODE_DISPATCH(CALL)
+#undef CALL
+}
+
+// ------------------------------------------------------------------------------------------
+// selected-block branch + sliding-window branch + gate in two launches
+extern "C" size_t nsa_decode_branches_gate_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                                           int64_t window_rows, int64_t topk, int64_t block_size) {
+  const size_t a = (decode_partial_bytes(batch, num_q_heads, num_kv_heads, head_dim, chunks_for(1, 0, topk, block_size)) + 255) & ~(size_t)255;
+  return a + decode_partial_bytes(batch, num_q_heads, num_kv_heads, head_dim, chunks_for(0, window_rows, 0, 64));
+}
+
+template <typename T, int D>
+static int run_branches_gate(DecodeParams& pa, DecodeParams& pb, const GateParams& g, char* ws, size_t bytes_a, hipStream_t s) {
+  const size_t na = (size_t)pa.B * pa.Hkv * pa.GT * pa.n_chunks * 16, nb = (size_t)pb.B * pb.Hkv * pb.GT * pb.n_chunks * 16;
+  pa.pm = (float*)ws; pa.pl = pa.pm + na; pa.po = pa.pl + na;
+  pb.pm = (float*)(ws + bytes_a); pb.pl = pb.pm + nb; pb.po = pb.pl + nb;
+  const int blocks_a = (pa.n_chunks + 3) / 4, blocks_b = (pb.n_chunks + 3) / 4;
+  decode_partial_pair_kernel<T, D><<<dim3((unsigned)(blocks_a + blocks_b), (unsigned)(pa.Hkv * pa.GT), (unsigned)pa.B), 256, 0, s>>>(pa, pb, blocks_a);
+  decode_merge_pair_gate_kernel<T, D><<<dim3((unsigned)(pa.Hkv * pa.G), (unsigned)pa.B), D <= 64 ? 64 : 128, 0, s>>>(pa, pb, g);
+  return nsa_check_launch();
+}
+
+extern "C" int nsa_decode_branches_gate(const void* q, const void* sparse_k, const void* sparse_v, const int32_t* sparse_len,
+                                        const int32_t* topk_idx, const void* window_k, const void* window_v, const int32_t* window_len,
+                                        const void* cmp_out, const void* gate, void* out, void* o_topk, void* o_window, int64_t batch,
+                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t sparse_rows,
+                                        int64_t window_rows, int64_t topk, int64_t block_size, const int64_t* strides, float sm_scale,
+                                        int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!strides) return NSA_ERR_BAD_ARG;
+  const int64_t sa[8] = {strides[0], strides[1], strides[2], strides[3], strides[4], strides[5], strides[6], strides[7]};
+  const int64_t sb[8] = {strides[0], strides[1], strides[11], strides[12], strides[13], strides[14], strides[15], strides[16]};
+  DecodeParams pa, pb;
+  int rc = fill_decode(pa, q, sparse_k, sparse_v, sparse_len, batch, num_q_heads, num_kv_heads, sparse_rows, sa, sm_scale);
+  if (rc != NSA_OK) return rc;
+  rc = fill_decode(pb, q, window_k, window_v, window_len, batch, num_q_heads, num_kv_heads, window_rows, sb, sm_scale);
+  if (rc != NSA_OK) return rc;
+  if (!topk_idx || !cmp_out || !gate || !out || !o_topk || !o_window || !workspace || topk <= 0) return NSA_ERR_BAD_ARG;
+  if (block_size != 32 && block_size != 64 && block_size != 128 && block_size != 256) return NSA_ERR_UNSUPPORTED;
+  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  if (workspace_bytes < nsa_decode_branches_gate_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, window_rows, topk, block_size))
+    return NSA_ERR_WORKSPACE;
+  pa.idx = topk_idx; pa.topk = (int)topk; pa.bs = (int)block_size;
+  pa.ish = strides[8]; pa.isb = strides[9]; pa.isk = strides[10];
+  pa.n_chunks = chunks_for(1, 0, topk, block_size);
+  pb.n_chunks = chunks_for(0, window_rows, 0, 64);
+  GateParams g;
+  g.cmp = cmp_out; g.gate = gate; g.out = out; g.o_a = o_topk; g.o_b = o_window;
+  g.csb = strides[17]; g.csh = strides[18]; g.gsb = strides[19]; g.gsh = strides[20]; g.gsk = strides[21];
+  g.osb = strides[22]; g.osh = strides[23]; g.asb = strides[24]; g.ash = strides[25]; g.bsb = strides[26]; g.bsh = strides[27];
+  const size_t bytes_a = (decode_partial_bytes(batch, num_q_heads, num_kv_heads, head_dim, pa.n_chunks) + 255) & ~(size_t)255;
+  hipStream_t s = (hipStream_t)stream;
+#define CALL(T, D) run_branches_gate<T, D>(pa, pb, g, (char*)workspace, bytes_a, s)
   DECODE_DISPATCH(CALL)
 #undef CALL
 }

@@ -21,6 +21,7 @@ from ..ops import (
     topk_sparse_attention_decode,
     weightedpool_compress,
 )
+from ..ops.decode import decode_branches_gate
 from ..ops.sliding_window import sliding_window_attention_varlen
 from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
 
@@ -186,9 +187,16 @@ def _decode_branches(cu_seqlens, step, query, key, value, gate_value, cache, ker
     """The three attention branches of a decode step over the updated cache, and their gated sum."""
     cmp_out, topk_idx = compressed_attention_infer(cu_seqlens, step, query, None, None, cache, kernel_size, kernel_stride, topk,
                                                    block_size, init_blocks, local_blocks)
-    sparse_out = topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size)
-    window_out = sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size)
-    out = gate_combine(gate_value, cmp_out, sparse_out, window_out)
+    batch = cu_seqlens.shape[0] - 1
+    if topk_idx.shape[-1] > 0 and gate_value.dtype == query.dtype:
+        # both remaining branches and the gate in two launches
+        out, sparse_out, window_out = decode_branches_gate(
+            query, cache.sparse_kv_cache[0, :batch], cache.sparse_kv_cache[1, :batch], cache.sparse_kv_len[:batch], topk_idx, block_size,
+            cache.sliding_kv_cache[0, :batch], cache.sliding_kv_cache[1, :batch], cache.sliding_kv_len[:batch], cmp_out, gate_value)
+    else:
+        sparse_out = topk_sparse_attention_infer(cu_seqlens, step, query, key, value, cache, topk_idx, block_size)
+        window_out = sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, window_size)
+        out = gate_combine(gate_value, cmp_out, sparse_out, window_out)
     if return_branches:
         return out, (cmp_out, sparse_out, window_out, topk_idx)
     return out

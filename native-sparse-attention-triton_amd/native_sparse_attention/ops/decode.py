@@ -44,7 +44,7 @@ def flash_attention_decode(q, k, v, seqlens, sm_scale: Optional[float] = None) -
     q, k, v = map(last_dim_contiguous, (q, k, v))
     o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     if L == 0:
-        return o
+        return o.zero_()
     lib = _lib.load()
     ws = _lib.workspace(lib.nsa_dense_decode_workspace_bytes(B, Hq, Hkv, D, L), q.device)
     rc = lib.nsa_dense_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), seqlens.data_ptr(), o.data_ptr(), B, Hq, Hkv, D, L,
@@ -65,7 +65,7 @@ def topk_sparse_attention_decode(q, k, v, topk_idx, block_size: int, seqlens, sm
     q, k, v = map(last_dim_contiguous, (q, k, v))
     o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     if L == 0 or topk == 0:
-        return o
+        return o.zero_()
     lib = _lib.load()
     ws = _lib.workspace(lib.nsa_topk_decode_workspace_bytes(B, Hq, Hkv, D, topk, block_size), q.device)
     rc = lib.nsa_topk_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), topk_idx.data_ptr(), seqlens.data_ptr(), o.data_ptr(),
@@ -109,3 +109,32 @@ def compressed_attention_decode(
                             ws.data_ptr(), ws.numel(), _lib.stream_ptr(q))
     _lib.check(rc, "nsa_cmp_decode")
     return o, idx
+
+
+def decode_branches_gate(q, sparse_k, sparse_v, sparse_len, topk_idx, block_size: int, window_k, window_v, window_len, cmp_out,
+                         gate_value, sm_scale: Optional[float] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """topk_sparse_attention_decode + flash_attention_decode over the sliding-window ring + the gated sum
+    gate[..., 0] * cmp_out + gate[..., 1] * selected + gate[..., 2] * window, as two kernel launches; the results are
+    those of the separate calls bit for bit.  Returns (gated sum, selected-branch output, window-branch output).
+    No counterpart of its own in the reference (it fuses infer/inference_func.py:140-202 and nsa_inference.py:146-150)."""
+    B, Hq, Hkv, D, L = _common_checks(q, sparse_k, sparse_v, sparse_len)
+    _, _, _, _, W = _common_checks(q, window_k, window_v, window_len)
+    assert Hkv == topk_idx.shape[0] and B == topk_idx.shape[1] and topk_idx.dtype == torch.int32
+    assert block_size in {32, 64, 128, 256} and L > 0 and W > 0 and topk_idx.shape[-1] > 0
+    assert cmp_out.shape == q.shape and gate_value.shape == (B, Hq, 3) and cmp_out.dtype == gate_value.dtype == q.dtype
+    topk = topk_idx.shape[-1]
+    if sm_scale is None:
+        sm_scale = 1 / math.sqrt(D)
+    q, sparse_k, sparse_v, window_k, window_v, cmp_out = map(last_dim_contiguous, (q, sparse_k, sparse_v, window_k, window_v, cmp_out))
+    out, o_sel, o_win = (torch.empty_like(q, memory_format=torch.contiguous_format) for _ in range(3))
+    lib = _lib.load()
+    ws = _lib.workspace(lib.nsa_decode_branches_gate_workspace_bytes(B, Hq, Hkv, D, W, topk, block_size), q.device)
+    strides = _lib.host_i64([q.stride(0), q.stride(1), *sparse_k.stride()[:3], *sparse_v.stride()[:3], *topk_idx.stride(),
+                             *window_k.stride()[:3], *window_v.stride()[:3], cmp_out.stride(0), cmp_out.stride(1), *gate_value.stride(),
+                             out.stride(0), out.stride(1), o_sel.stride(0), o_sel.stride(1), o_win.stride(0), o_win.stride(1)])
+    rc = lib.nsa_decode_branches_gate(q.data_ptr(), sparse_k.data_ptr(), sparse_v.data_ptr(), sparse_len.data_ptr(), topk_idx.data_ptr(),
+                                      window_k.data_ptr(), window_v.data_ptr(), window_len.data_ptr(), cmp_out.data_ptr(),
+                                      gate_value.data_ptr(), out.data_ptr(), o_sel.data_ptr(), o_win.data_ptr(), B, Hq, Hkv, D, L, W, topk,
+                                      block_size, strides, sm_scale, _lib.dtype_code(q), ws.data_ptr(), ws.numel(), _lib.stream_ptr(q))
+    _lib.check(rc, "nsa_decode_branches_gate")
+    return out, o_sel, o_win
