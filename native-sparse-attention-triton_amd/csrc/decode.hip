@@ -246,9 +246,12 @@ struct ScoreParams {
   int B, Hkv, G, GT, slab_len, ks, st, bs, init_blocks, local_blocks, k_out, max_blocks, full_blocks;
   long long qsb, qsh, ksb, ksn, ksh, osh, osb, osk;
   float qk_scale;
+  // merge of the attention partials, done here when selection follows (one launch less, and the LSE never
+  // leaves the chip): partials as in DecodeParams, o = attention output [B, Hq, D]
+  const float* pm; const float* pl; const float* po; int n_chunks; void* o; long long oob, ooh;
 };
 
-static constexpr int MAX_SCORE_BLOCKS = 8192;
+static constexpr int MAX_SCORE_BLOCKS = 8192, MAX_SCORE_GROUP = 128;
 
 // One workgroup of SEL_NT threads per (kv-head, sequence): the work is a chain of short dependent phases, so
 // the aim is few round trips to memory and few barriers, not throughput.
@@ -268,7 +271,40 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
   const int qb = (p.seqlens[b] - 1) / p.bs;
   // per-key scores stay in LDS when they fit (a round trip to memory less), else in the workspace
   __shared__ float score_s[SEL_LDS_SCORES];
+  __shared__ float lse_s[MAX_SCORE_GROUP];
   float* score = lc <= SEL_LDS_SCORES ? score_s : p.score + ((long long)b * p.Hkv + h) * p.slab_len;
+  // phase 0: merge the chunk partials of this kv-head's query heads, one wave per head: the lanes share out
+  // the chunks for the maximum and the sum, then each lane owns output columns lane, lane + 64
+  for (int hq = wave; hq < p.G; hq += SEL_NW) {
+    const int col = hq % 16;
+    const long long base = (((long long)b * p.Hkv + h) * p.GT + hq / 16) * p.n_chunks;
+    float m = -INFINITY;
+    for (int c = lane; c < p.n_chunks; c += 64) m = fmaxf(m, p.pm[(base + c) * 16 + col]);
+    m = wave_max_f32(m);
+    float l = 0.f;
+    for (int c = lane; c < p.n_chunks; c += 64) {
+      const float mc = p.pm[(base + c) * 16 + col];
+      if (mc != -INFINITY) l += fast_exp2(mc - m) * p.pl[(base + c) * 16 + col];
+    }
+    l = wave_sum_f32(l);
+    float acc[(D + 63) / 64];
+#pragma unroll
+    for (int u = 0; u < (D + 63) / 64; u++) acc[u] = 0.f;
+#pragma unroll 4
+    for (int c = 0; c < p.n_chunks; c++) {
+      const float mc = p.pm[(base + c) * 16 + col];
+      const float w = mc != -INFINITY ? fast_exp2(mc - m) : 0.f;
+#pragma unroll
+      for (int u = 0; u < (D + 63) / 64; u++)
+        if (lane + 64 * u < D) acc[u] += p.po[((base + c) * 16 + col) * D + lane + 64 * u] * w;
+    }
+    T* orow = (T*)p.o + (long long)b * p.oob + (long long)(h * p.G + hq) * p.ooh;
+#pragma unroll
+    for (int u = 0; u < (D + 63) / 64; u++)
+      if (lane + 64 * u < D) orow[lane + 64 * u] = (T)(l > 0.f ? acc[u] / l : 0.f);
+    if (lane == 0) lse_s[hq] = l > 0.f ? m + fast_log2(l) : INFINITY;
+  }
+  __syncthreads();
   // phase A: score[c] = sum over the group's heads of exp2(s*scale - lse); a wave takes two 16-key tiles per
   // trip and issues the K loads of both before it uses either
   for (int sub0 = 2 * wave; sub0 * 16 < lc; sub0 += 2 * SEL_NW) {
@@ -286,7 +322,7 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
       const int hq = gt * 16 + li;
       const bool has_head = hq < p.G;
       const T* qp = (const T*)p.q + (long long)b * p.qsb + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
-      const float l2 = has_head ? p.lse[(long long)b * p.Hkv * p.G + h * p.G + hq] : INFINITY;
+      const float l2 = has_head ? lse_s[hq] : INFINITY;
       v8 qf[NK];
 #pragma unroll
       for (int kk = 0; kk < NK; kk++) qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
@@ -466,12 +502,14 @@ template <typename T, int D>
 static int run_cmp_decode(DecodeParams& p, ScoreParams& sp, void* o, long long osb, long long osh, char* ws, size_t part_bytes, hipStream_t s) {
   float* lse = (float*)(ws + part_bytes);
   float* score = (float*)(ws + part_bytes + (((size_t)p.B * p.Hkv * p.G * 4 + 255) & ~(size_t)255));
-  int rc = run_decode<T, D>(0, p, o, osb, osh, lse, ws, s);
-  if (rc != NSA_OK) return rc;
-  if (sp.out_idx) {
-    sp.lse = lse; sp.score = score;
-    decode_score_select_kernel<T, D><<<dim3((unsigned)p.Hkv, (unsigned)p.B), SEL_NT, 0, s>>>(sp);
-  }
+  if (!sp.out_idx) return run_decode<T, D>(0, p, o, osb, osh, lse, ws, s);
+  // with selection: partials, then one kernel that merges them, scores the blocks and picks
+  const size_t n = (size_t)p.B * p.Hkv * p.GT * p.n_chunks * 16;
+  p.pm = (float*)ws; p.pl = p.pm + n; p.po = p.pl + n;
+  decode_partial_kernel<T, D, 0><<<dim3((unsigned)((p.n_chunks + 3) / 4), (unsigned)(p.Hkv * p.GT), (unsigned)p.B), 256, 0, s>>>(p);
+  sp.lse = lse; sp.score = score;
+  sp.pm = p.pm; sp.pl = p.pl; sp.po = p.po; sp.n_chunks = p.n_chunks; sp.o = o; sp.oob = osb; sp.ooh = osh;
+  decode_score_select_kernel<T, D><<<dim3((unsigned)p.Hkv, (unsigned)p.B), SEL_NT, 0, s>>>(sp);
   return nsa_check_launch();
 }
 
@@ -488,7 +526,7 @@ extern "C" int nsa_cmp_decode(const void* q, const void* k, const void* v, const
   if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
   if (workspace_bytes < nsa_cmp_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, slab_len)) return NSA_ERR_WORKSPACE;
   const int64_t max_blocks = (max_seqlen + block_size - 1) / block_size;
-  if (out_topk_idx && (k_out <= 0 || k_out > 64 || k_out > max_blocks || max_blocks > MAX_SCORE_BLOCKS)) return NSA_ERR_UNSUPPORTED;
+  if (out_topk_idx && (k_out <= 0 || k_out > 64 || k_out > max_blocks || max_blocks > MAX_SCORE_BLOCKS || p.G > MAX_SCORE_GROUP)) return NSA_ERR_UNSUPPORTED;
   p.n_chunks = chunks_for(0, slab_len, 0, 64);
   ScoreParams sp;
   sp.q = q; sp.k = k; sp.seqlens = seqlens; sp.clens = compress_seqlens; sp.out_idx = out_topk_idx;
