@@ -48,10 +48,12 @@ class NSADecodeGraph:
     @torch.no_grad()
     def step(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, gate_value: torch.Tensor) -> torch.Tensor:
         """One new token per sequence; returns a view of the graph's output buffer (valid until the next call)."""
-        self.query.copy_(query)
-        self.key.copy_(key)
-        self.value.copy_(value)
-        self.gate.copy_(gate_value)
+        dst, src = [self.query, self.key, self.value, self.gate], [query, key, value, gate_value]
+        if hasattr(torch, "_foreach_copy_"):
+            torch._foreach_copy_(dst, src)   # one launch for the four copies
+        else:
+            for d, s in zip(dst, src):
+                d.copy_(s)
         self.graph.replay()
         return self.out
 
