@@ -3,10 +3,12 @@
 //   top-k      - the 64-token-aligned blocks named by topk_idx[h, b, :]
 //   compressed - dense over the compressed slab, then per-key probabilities summed over the GQA
 //                group -> overlap-weighted block scores -> forced init/local blocks -> top-k ids
-// All three share one split-K kernel: a workgroup takes 64 keys of one (sequence, kv-head), each
-// wave 16 of them, with the (up to 16) query heads of the group as MFMA columns; partial
-// (max, sum, O) triples go to the workspace and a second kernel merges them.  The work is a few
-// MiB per step, so the aim is few launches and coalesced 16-byte accesses, not MFMA rate.
+// All three share one split-K body: a wave takes a chunk of up to 64 keys of one (sequence, kv-head) with the
+// (up to 16) query heads of the group as MFMA columns and writes a partial (max, sum, O) triple to the
+// workspace; a second kernel merges the partials.  The work is a few MiB per step, so the aim is few launches,
+// few dependent round trips to memory and no barriers, not MFMA rate.  For a whole decode step the
+// selected-block and the sliding-window branch share one partial launch, and one launch does both merges and
+// the gated sum with the compressed branch; the compressed branch's merge runs inside its block-selection kernel.
 #include "nsa_common.h"
 
 struct DecodeParams {
