@@ -19,6 +19,7 @@
 
 struct CmpParams {
   const void* q; const void* k; const void* v; const void* dout; void* o; void* dq; float* lse; const float* delta;
+  float* delta_out;  // backward dQ: when set, delta = rowsum(o * dout) is formed there (from the dO rows it holds) and stored here
   const int32_t* cu_q; const int32_t* cu_k;
   int total_q, batch, Hkv, G, GT, ks, st;
   int window;  // -1: compressed keys (rule above); >= 0: ordinary keys, position i sees j in [i - window, i]; -2: ordinary keys, all visible
@@ -339,7 +340,20 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
       dof[j][kk] = live ? ld16<v8>(dp + 32 * kk) : zero16<v8>();
     }
     l2[j] = live ? p.lse[(long long)hh * p.total_q + t] : INFINITY;
-    dl[j] = live ? p.delta[(long long)hh * p.total_q + t] : 0.f;
+    if (p.delta_out) {
+      const T* op = (const T*)p.o + t * p.osn + (long long)hh * p.osh + 8 * lg;
+      float part = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) {
+        const v8 of = live ? ld16<v8>(op + 32 * kk) : zero16<v8>();
+#pragma unroll
+        for (int e = 0; e < 8; e++) part = __builtin_fmaf((float)of[e], (float)dof[j][kk][e], part);
+      }
+      dl[j] = column_sum(part);
+      if (live && lg == 0) p.delta_out[(long long)hh * p.total_q + t] = dl[j];
+    } else {
+      dl[j] = live ? p.delta[(long long)hh * p.total_q + t] : 0.f;
+    }
   }
   int tile_lo, tile_hi, unused;
   visible_range(min(ti.i0 + 7, ti.lq - 1), ti.lq, ti.lk, p.ks, p.st, p.window, unused, tile_hi);
@@ -701,7 +715,9 @@ static int run_cmp(CmpArgs& a) {
     int32_t* seg_end = (int32_t*)(a.ws + L.seg_end);
     int32_t* chunk_off = (int32_t*)(a.ws + L.chunk_off);
     const int n_seg = (int)(a.Hkv * L.max_blocks);
-    launch_delta<T, D>((const T*)a.o_in, (const T*)a.p.dout, delta, a.Tq, a.Hq, a.p.osn, a.p.osh, a.p.dsn, a.p.dsh, a.stream);
+    // dQ first: it forms delta = rowsum(O * dO) from the dO rows it holds and leaves it behind for the dK/dV pass
+    a.p.o = const_cast<void*>(a.o_in); a.p.delta = nullptr; a.p.delta_out = delta;
+    cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
     cmp_segments_kernel<<<1, 64, 0, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
     chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off);
     DkdvParams d;
@@ -716,8 +732,6 @@ static int run_cmp(CmpArgs& a) {
     else dkdv_kernel<T, D, 64, true, false><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
     dkdv_reduce_kernel<T, D, 64><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
                                                                        (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
-    a.p.delta = delta;
-    cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
   }
   return nsa_check_launch();
 }
@@ -747,7 +761,7 @@ static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, c
   p.G = (int)(Hq / Hkv); p.GT = (p.G + 15) / 16; p.ks = (int)ks; p.st = (int)st;
   p.qsn = strides[0]; p.qsh = strides[1]; p.ksn = strides[2]; p.ksh = strides[3]; p.vsn = strides[4]; p.vsh = strides[5];
   p.qk_scale = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale; p.window = -1;
-  p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr;
+  p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr; p.delta_out = nullptr;
   a.Tq = Tq; a.Tk = Tk; a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.stream = (hipStream_t)stream; a.ws = nullptr;
   return NSA_OK;
 }
