@@ -666,14 +666,16 @@ __global__ void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int3
   }
 }
 
-struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, partial, total; int64_t max_blocks, max_items; };
+struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, partial, total; int64_t max_blocks, max_items; int chunk; };
 static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
   CmpBwdLayout L;
   L.max_blocks = Tk / 64 + B;
   const int64_t GT = (Hq / Hkv + 15) / 16;
   (void)GT;
-  // every block's range is at most Tq tokens: ceil(Tq/CHUNK)+1 items per segment is a safe bound
-  L.max_items = Hkv * L.max_blocks * ((Tq + CHUNK_TOKENS - 1) / CHUNK_TOKENS + 1);
+  // queries per work item from a bound on the (query, key block) pairs (a causal range covers about half of Tq);
+  // every block's range is at most Tq tokens: ceil(Tq/chunk)+1 items per segment is a safe bound
+  L.chunk = dkdv_chunk_tokens(Hkv * L.max_blocks * Tq / 2);
+  L.max_items = Hkv * L.max_blocks * ((Tq + L.chunk - 1) / L.chunk + 1);
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
   L.delta = take((size_t)Hq * Tq * 4);
@@ -719,13 +721,13 @@ static int run_cmp(CmpArgs& a) {
     a.p.o = const_cast<void*>(a.o_in); a.p.delta = nullptr; a.p.delta_out = delta;
     cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
     cmp_segments_kernel<<<1, 64, 0, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
-    chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off);
+    chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off, L.chunk);
     DkdvParams d;
     d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
     d.cu_blk = cu_blk; d.seg_begin = seg_begin; d.seg_end = seg_end; d.chunk_off = chunk_off; d.queries = nullptr;
     d.partial = (float*)(a.ws + L.partial);
     d.total_len = (int)a.Tq; d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;
-    d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st; d.window = a.p.window;
+    d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st; d.window = a.p.window; d.chunk = L.chunk;
     d.qsn = (int)a.p.qsn; d.qsh = (int)a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = (int)a.p.dsn; d.dsh = (int)a.p.dsh;
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
     if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);

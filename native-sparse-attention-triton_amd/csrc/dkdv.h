@@ -4,7 +4,7 @@
 // MFMA B operands, and streams query rows through double-buffered LDS two (token, head-tile) row
 // groups at a time.  P and dS leave the score MFMA already in B-operand layout; the transposed
 // Q and dO fragments are read from LDS with ds_read_b64_tr_b16.  Work items are (segment,
-// chunk of CHUNK_TOKENS queries); each writes an fp32 partial, a second kernel adds the chunks of
+// chunk of up to MAX_CHUNK_TOKENS queries); each writes an fp32 partial, a second kernel adds the chunks of
 // a segment in order, so no atomics are needed and results are reproducible.
 //   RANGE = false: the queries of a segment come from a sorted list (reverse index of topk_idx),
 //                  key j is visible to a query at position pos iff j <= pos.
@@ -13,7 +13,16 @@
 #pragma once
 #include "nsa_common.h"
 
-static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
+static constexpr int MAX_CHUNK_TOKENS = 1024;  // most queries per dK/dV work item
+
+// Queries per work item, from the number of (query, key block) pairs of the launch: long items amortise the
+// loading of K/V and the partial they write, but a launch needs a few thousand items to fill 256 CUs three
+// workgroups deep and to even out the one segment every token selects (its chunks are the longest items).
+static inline int dkdv_chunk_tokens(long long pairs) {
+  if (pairs >= 2048ll * 1024) return 1024;
+  if (pairs >= 2048ll * 512) return 512;
+  return 256;
+}
 
 // Waves per dK/dV workgroup; each wave owns bs / (16 * waves) key tiles.  Every wave reads all staged
 // query rows from LDS, so fewer waves would mean fewer LDS reads per token, but 32 keys per wave need 192
@@ -23,15 +32,15 @@ static constexpr int CHUNK_TOKENS = 1024;  // queries per dK/dV work item
 // wave at three waves per SIMD.
 constexpr int dkdv_waves(int bs) { return bs >= 64 ? 4 : bs / 16; }
 
-// chunk_off = exclusive scan of ceil((seg_end - seg_begin)/CHUNK_TOKENS) over segments (single workgroup).
+// chunk_off = exclusive scan of ceil((seg_end - seg_begin)/chunk) over segments (single workgroup).
 static __global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* __restrict__ seg_begin, const int32_t* __restrict__ seg_end, int n_seg,
-                                                          int32_t* __restrict__ chunk_off) {
+                                                          int32_t* __restrict__ chunk_off, int chunk) {
   __shared__ int part[1024];
   const int tid = threadIdx.x;
   const int per = (n_seg + 1023) / 1024;
   const int j0 = tid * per, j1 = min(n_seg, j0 + per);
   int s = 0;
-  for (int j = j0; j < j1; j++) s += (seg_end[j] - seg_begin[j] + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
+  for (int j = j0; j < j1; j++) s += (seg_end[j] - seg_begin[j] + chunk - 1) / chunk;
   part[tid] = s;
   __syncthreads();
   for (int d = 1; d < 1024; d <<= 1) {
@@ -43,7 +52,7 @@ static __global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* 
   int run = part[tid] - s;
   for (int j = j0; j < j1; j++) {
     chunk_off[j] = run;
-    run += (seg_end[j] - seg_begin[j] + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
+    run += (seg_end[j] - seg_begin[j] + chunk - 1) / chunk;
   }
   if (tid == 1023) chunk_off[n_seg] = part[1023];
 }
@@ -53,6 +62,7 @@ struct DkdvParams {
   const int32_t* cu; const int32_t* cu_k; const int32_t* cu_blk; const int32_t* seg_begin; const int32_t* seg_end; const int32_t* chunk_off; const int32_t* queries;
   float* partial;
   int total_len, batch, Hkv, G, GT, max_blocks, n_seg, ks, st;
+  int chunk;   // queries per work item (dkdv_chunk_tokens)
   int window;  // range mode: -1 compressed keys (key c seen from position c*st + ks - 1 on), >= 0 ordinary keys seen by [key, key + window], -2 every key seen by every position
   long long ksn, ksh, vsn, vsh;
   int qsn, qsh, dsn, dsh;  // element strides of q / dO (dkdv_strides_fit() on the host)
@@ -111,8 +121,8 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 3 : 1) void dkdv_ke
   const int s0 = p.cu[b];                                  // first query token of the sequence
   const int k0 = p.cu_k[b], len = p.cu_k[b + 1] - k0;      // its keys
   const int key0 = (gb - p.cu_blk[b]) * BS;
-  const int first = p.seg_begin[seg] + (item - p.chunk_off[seg]) * CHUNK_TOKENS;
-  const int n_tok = min(CHUNK_TOKENS, p.seg_end[seg] - first);
+  const int first = p.seg_begin[seg] + (item - p.chunk_off[seg]) * p.chunk;
+  const int n_tok = min(p.chunk, p.seg_end[seg] - first);
   const int GT = GT1 ? 1 : p.GT;
   const int n_rg = n_tok * GT;                // row groups (token, head tile) in this chunk
   const int n_step = (n_rg + 1) / 2;
@@ -139,7 +149,7 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 3 : 1) void dkdv_ke
 
   // token ids of this chunk, read once (list mode): the source addresses of a step then need no
   // global load of their own
-  __shared__ int tok_s[CHUNK_TOKENS];
+  __shared__ int tok_s[MAX_CHUNK_TOKENS];
   for (int i = tid; i < n_tok; i += NT) tok_s[i] = RANGE ? first + i : p.queries[first + i];
   __syncthreads();
 
