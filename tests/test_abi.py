@@ -67,3 +67,29 @@ def test_backward_refuses_strides_beyond_31_bits():
     rc = lib.nsa_topk_attn_bwd(fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, 2048, 1, 64, 4, 128, 16, 64, strides, 0.1,
                                0, fake, ws, None, None, 7, None)
     assert rc == -2
+
+
+def test_decode_step_entry_points_check_their_arguments():
+    lib = _lib.load()
+    fake = 1 << 20
+    strides8 = (ctypes.c_int64 * 8)(4096, 128, 256, 128, 256, 128, 4096, 128)
+    # a null slab pointer
+    rc = lib.nsa_decode_prepare(fake, fake, fake, fake, None, None, None, fake, 1.0, None, fake, fake, fake, fake, fake, fake, fake,
+                                4, 32, 2, 128, strides8, 4, 32, 16, 511, 8192, 512, 0, None)
+    assert rc == -1
+    # more sequences than the slabs hold
+    rc = lib.nsa_decode_prepare(fake, fake, fake, fake, None, None, None, fake, 1.0, fake, fake, fake, fake, fake, fake, fake, fake,
+                                5, 32, 2, 128, strides8, 4, 32, 16, 511, 8192, 512, 0, None)
+    assert rc == -1
+    # a row stride that is not a multiple of 8 elements
+    bad = (ctypes.c_int64 * 8)(4100, 128, 256, 128, 256, 128, 4096, 128)
+    rc = lib.nsa_decode_prepare(fake, fake, fake, fake, None, None, None, fake, 1.0, fake, fake, fake, fake, fake, fake, fake, fake,
+                                4, 32, 2, 128, bad, 4, 32, 16, 511, 8192, 512, 0, None)
+    assert rc == -2
+    # the two-launch branches + gate call: workspace too small
+    strides28 = (ctypes.c_int64 * 28)(*([128] * 28))
+    need = lib.nsa_decode_branches_gate_workspace_bytes(4, 32, 2, 128, 512, 8, 64)
+    assert need > 0
+    rc = lib.nsa_decode_branches_gate(fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, 4, 32, 2, 128, 8192, 512,
+                                      8, 64, strides28, 0.088, 0, fake, need - 1, None)
+    assert rc == -3
