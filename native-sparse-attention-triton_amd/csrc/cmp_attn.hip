@@ -217,7 +217,10 @@ __global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams 
           mloc = fmaxf(mloc, s[j][sub][r]);
         }
       mloc = column_max(mloc);
-      const float m_new = fmaxf(m[j], mloc);
+      // the reference maximum only moves when a chunk beats it by more than RESCALE_SLACK in the exponent:
+      // until then probabilities are formed against the old reference (at most 2^RESCALE_SLACK: exact in
+      // the fp32 sums, within range of bf16/fp16) and alpha stays exactly 1, so the rescale below is skipped
+      const float m_new = (mloc - m[j]) * p.qk_scale > RESCALE_SLACK ? mloc : m[j];
       alpha[j] = fast_exp2((m[j] - m_new) * p.qk_scale);
       const float mb = m_new * p.qk_scale;
       m[j] = m_new;
