@@ -30,7 +30,7 @@ static inline int dkdv_chunk_tokens(long long pairs) {
 // and at one wave per SIMD (with the score and the dK/dV MFMAs of neighbouring steps interleaved by
 // hand) the single wave's instruction issue became the limit - both measured slower than one tile per
 // wave at three waves per SIMD.
-constexpr int dkdv_waves(int bs) { return bs >= 64 ? 4 : bs / 16; }
+constexpr int dkdv_waves(int bs) { return bs >= 256 ? 8 : (bs >= 64 ? 4 : bs / 16); }
 
 // chunk_off = exclusive scan of ceil((seg_end - seg_begin)/chunk) over segments (single workgroup).
 static __global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* __restrict__ seg_begin, const int32_t* __restrict__ seg_end, int n_seg,
