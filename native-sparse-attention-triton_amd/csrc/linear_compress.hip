@@ -70,39 +70,40 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(LinParams p) {
   f32x4 acc[NET];
 #pragma unroll
   for (int i = 0; i < NET; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // W tile staging registers.  The loads and the LDS writes are written out at their three places of use:
+  // as lambdas over a register array the array ended up in scratch memory.
   uint4 regs[PPT];
-  auto fetch = [&](int step) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * 256;
-      if (pc < PIECES) regs[u] = *reinterpret_cast<const uint4*>(wh + ((long long)step * 32 + pc / (D / 8)) * D + (pc % (D / 8)) * 8);
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < PPT; u++) {
-      const int pc = tid + u * 256;
-      if (pc < PIECES) *reinterpret_cast<uint4*>(&w_s[buf][pc / (D / 8)][(pc % (D / 8)) * 8]) = regs[u];
-    }
-  };
+#define LIN_FETCH(STEP)                                                                                              \
+  _Pragma("unroll") for (int u = 0; u < PPT; u++) {                                                                  \
+    const int pc = min(tid + u * 256, PIECES - 1);                                                                   \
+    regs[u] = *reinterpret_cast<const uint4*>(wh + ((long long)(STEP) * 32 + pc / (D / 8)) * D + (pc % (D / 8)) * 8); \
+  }
+#define LIN_STASH(BUF)                                                                                               \
+  _Pragma("unroll") for (int u = 0; u < PPT; u++) {                                                                  \
+    const int pc = tid + u * 256;                                                                                    \
+    if (pc < PIECES) *reinterpret_cast<uint4*>(&w_s[BUF][pc / (D / 8)][(pc % (D / 8)) * 8]) = regs[u];               \
+  }
   // step = (k, 32-wide slice of d): rows [32*step, +32) of W[h]; blockIdx.z takes a contiguous share of the steps
   const int all_steps = p.ks * NK, per = (all_steps + p.splits - 1) / p.splits;
   const int step0 = blockIdx.z * per, n_steps = min(all_steps, step0 + per);
   if (step0 < n_steps) {
-    fetch(step0);
-    stash(step0 & 1);
+    LIN_FETCH(step0)
+    LIN_STASH(step0 & 1)
   }
   __syncthreads();
   for (int step = step0; step < n_steps; step++) {
     const int buf = step & 1;
-    if (step + 1 < n_steps) fetch(step + 1);
+    const int nxt = min(step + 1, n_steps - 1);   // the last trip loads its own tile again and does not store it
+    LIN_FETCH(nxt)
     const int k = step / NK, c = step % NK;
     const v8 xf = row_frag<T>(xrow + (long long)k * p.xsn, 32 * c, lg, live);
 #pragma unroll
     for (int et = 0; et < NET; et++) acc[et] = E::mfma16(lds_tr_frag<T, LD>(w_s[buf], 16 * et, li, lg), xf, acc[et]);
-    if (step + 1 < n_steps) stash(buf ^ 1);
+    if (step + 1 < n_steps) { LIN_STASH(buf ^ 1) }
     __syncthreads();
   }
+#undef LIN_FETCH
+#undef LIN_STASH
   if (live && p.splits == 1) {
     T* yp = (T*)p.y + (long long)(p.ycu[b] + n) * p.ysn + (long long)h * p.ysh + 4 * lg;
 #pragma unroll
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(256) void lin_dw_kernel(LinParams p) {
     for (int i = 0; i < NET; i++) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
   constexpr int PIECES1 = 32 * (D / 8), PPT1 = (PIECES1 + 255) / 256;  // per tensor
   uint4 rx[PPT1], rg[PPT1];
-  auto fetch = [&](int chunk) {
+  auto fetch = [&](int chunk) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < PPT1; u++) {
       const int pc = tid + u * 256;
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(256) void lin_dw_kernel(LinParams p) {
       rg[u] = vg;
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < PPT1; u++) {
       const int pc = tid + u * 256;
