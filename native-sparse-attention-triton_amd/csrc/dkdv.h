@@ -86,9 +86,10 @@ static inline bool dkdv_strides_fit(long long qsn, long long qsh, long long dsn,
   return qsn >= 0 && dsn >= 0 && qsh >= 0 && dsh >= 0 && qsn <= lim && dsn <= lim && G * qsh + D <= lim && G * dsh + D <= lim;
 }
 
-// GT1: the GQA group has at most 16 query heads (one head tile), which removes every run-time division
+// GT1: the GQA group has at most 16 query heads (one head tile), which removes every run-time division.
+// The workgroups-per-CU hint is the largest for which the variant compiles without register spills.
 template <typename T, int D, int BS, bool RANGE, bool GT1>
-__global__ __launch_bounds__(64 * dkdv_waves(BS), BS <= 64 ? 3 : 1) void dkdv_kernel(DkdvParams p) {
+__global__ __launch_bounds__(64 * dkdv_waves(BS), BS == 64 ? (GT1 ? 3 : 2) : (BS < 64 ? (D >= 96 ? 3 : 2) : 1)) void dkdv_kernel(DkdvParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32, NDT = D / 16, NSUB = BS / 16;
