@@ -677,7 +677,7 @@ static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq
   (void)GT;
   // queries per work item from a bound on the (query, key block) pairs (a causal range covers about half of Tq);
   // every block's range is at most Tq tokens: ceil(Tq/chunk)+1 items per segment is a safe bound
-  L.chunk = dkdv_chunk_tokens(Hkv * L.max_blocks * Tq / 2);
+  L.chunk = dkdv_chunk_tokens(Hkv * L.max_blocks * Tq / 2, MAX_CHUNK_TOKENS);
   L.max_items = Hkv * L.max_blocks * ((Tq + L.chunk - 1) / L.chunk + 1);
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };

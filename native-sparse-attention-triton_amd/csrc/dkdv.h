@@ -13,13 +13,17 @@
 #pragma once
 #include "nsa_common.h"
 
-static constexpr int MAX_CHUNK_TOKENS = 1024;  // most queries per dK/dV work item
+// Most queries per dK/dV work item.  The token list of an item lives in LDS next to the three staging
+// buffers; with 960 entries a d = 128 workgroup needs 53760 bytes, the most for which three workgroups
+// share a CU's 160 KiB (with 1024 entries only two were resident and the pass ran 8 % slower).
+static constexpr int MAX_CHUNK_TOKENS = 960;
 
 // Queries per work item, from the number of (query, key block) pairs of the launch: long items amortise the
 // loading of K/V and the partial they write, but a launch needs a few thousand items to fill 256 CUs three
 // workgroups deep and to even out the one segment every token selects (its chunks are the longest items).
-static inline int dkdv_chunk_tokens(long long pairs) {
-  if (pairs >= 2048ll * 1024) return 1024;
+// `longest` is the size used by big launches (measured best: 768 for query lists, 960 for query ranges).
+static inline int dkdv_chunk_tokens(long long pairs, int longest) {
+  if (pairs >= 2048ll * 1024) return longest < MAX_CHUNK_TOKENS ? longest : MAX_CHUNK_TOKENS;
   if (pairs >= 2048ll * 512) return 512;
   return 256;
 }

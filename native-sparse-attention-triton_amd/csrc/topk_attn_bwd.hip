@@ -26,6 +26,8 @@ struct BwdLayout {
   int64_t max_blocks, n_pairs, max_items, n_slots;
 };
 
+static constexpr int LIST_CHUNK = 768;  // queries per dK/dV work item in big launches
+
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t topk, int64_t bs) {
@@ -33,7 +35,7 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.max_blocks = T / bs + B;  // every sequence adds at most one ragged block
   L.n_pairs = Hkv * T * topk;
   const int64_t GT = (Hq / Hkv + 15) / 16;
-  const int chunk = dkdv_chunk_tokens(L.n_pairs);
+  const int chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
   L.max_items = (L.n_pairs + chunk - 1) / chunk + Hkv * L.max_blocks;
   (void)GT;
   size_t tmp = 0;
@@ -289,7 +291,7 @@ static int build_reverse_index(const BwdArgs& a, const BwdLayout& L) {
   if (rocprim::radix_sort_pairs(ws + L.sort_tmp, tmp, keys_in, keys_out, vals_in, vals_out, (size_t)L.n_pairs, 0u, bits, a.stream) != hipSuccess)
     return NSA_ERR_LAUNCH;
   segment_offsets_kernel<<<(n_seg + 1 + 255) / 256, 256, 0, a.stream>>>(keys_out, L.n_pairs, n_seg, seg_off);
-  chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_off, seg_off + 1, n_seg, chunk_off, dkdv_chunk_tokens(L.n_pairs));
+  chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_off, seg_off + 1, n_seg, chunk_off, dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK));
   return nsa_check_launch();
 }
 
@@ -338,7 +340,7 @@ static int run_bwd(const BwdArgs& a) {
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
     p.qsn = (int)a.qsn; p.qsh = (int)a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = (int)a.dsn; p.dsh = (int)a.dsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1; p.window = -1;
-    p.chunk = dkdv_chunk_tokens(L.n_pairs);
+    p.chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
     constexpr int NT = 64 * dkdv_waves(BS);
     if (GT == 1) dkdv_kernel<T, D, BS, false, true><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
     else dkdv_kernel<T, D, BS, false, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
