@@ -447,6 +447,7 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
 struct SelParams {
   const void* q; const void* k; const float* lse; const int32_t* cu_q; const int32_t* cu_k; int32_t* out;
   int total_q, batch, Hkv, G, GT, ks, st, bs, init_blocks, local_blocks, k_out, nb_cap, full_blocks;
+  int nb_lo, nb_row;  // this launch takes the tiles that need nb_lo < blocks <= nb_row score entries per token; nb_row is the row pitch
   long long qsn, qsh, ksn, ksh, osh, osn, osk;
   float qk_scale;
 };
@@ -468,13 +469,18 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
   constexpr int NK = D / 32, LD = lds_pitch(D);
   __shared__ __attribute__((aligned(16))) T k_s[2][32][LD];
   extern __shared__ float dyn[];
-  float* bs_s = dyn;                           // [16][nb_cap] block scores of the tile's tokens
+  float* bs_s = dyn;                           // [16][nb_row] block scores of the tile's tokens
   TileInfo ti;
   if (!locate_tile(p.cu_q, p.cu_k, p.batch, blockIdx.x, ti)) return;
+  const int tile_last = min(ti.i0 + 15, ti.lq - 1);
+  {  // tiles are shared out over launches by the number of blocks their last token can choose from
+    const int need = min(tile_last / p.bs + 1, p.nb_cap);
+    if (need <= p.nb_lo || need > p.nb_row) return;
+  }
   const int h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), li = lane & 15, lg = lane >> 4;
   const int a = A ? A : p.ks / p.st, rr = A ? RR : p.bs / p.st;  // keys per kernel window and per selection block
-  for (int i = tid; i < 16 * p.nb_cap; i += 256) bs_s[i] = 0.f;
+  for (int i = tid; i < 16 * p.nb_row; i += 256) bs_s[i] = 0.f;
   int lim[4];
   int wave_lim = 0, wave_lim_min = 1 << 30;
 #pragma unroll
@@ -483,7 +489,6 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
     wave_lim = max(wave_lim, lim[j]);
     wave_lim_min = min(wave_lim_min, lim[j]);
   }
-  const int tile_last = min(ti.i0 + 15, ti.lq - 1);
   const int n_chunks = (visible_keys(tile_last, ti.lq, ti.lk, p.ks, p.st) + 31) / 32;
   const T* kb = (const T*)p.k + (long long)ti.k0 * p.ksn + (long long)h * p.ksh;
   Stager<T, D, 1> stg;
@@ -563,8 +568,8 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
           }
           xprev = xs;
           const int blk = c / rr;
-          if ((li & (min(rr, 16) - 1)) == 0 && blk < p.full_blocks && blk < p.nb_cap)
-            atomicAdd(&bs_s[(4 * wave + lg) * p.nb_cap + blk], z);  // LDS add without return: nothing waits for it
+          if ((li & (min(rr, 16) - 1)) == 0 && blk < p.full_blocks && blk < p.nb_row)
+            atomicAdd(&bs_s[(4 * wave + lg) * p.nb_row + blk], z);  // LDS add without return: nothing waits for it
         }
       }
       if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], k_s[buf ^ 1], tid);
@@ -575,9 +580,9 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
   for (int j = 0; j < 4; j++) {
     const int pos = ti.i0 + 4 * wave + j;
     if (pos >= ti.lq) continue;  // wave-uniform
-    float* row = bs_s + (4 * wave + j) * p.nb_cap;
+    float* row = bs_s + (4 * wave + j) * p.nb_row;
     const int qb = pos / p.bs;
-    const int nb = min(qb + 1, p.nb_cap);
+    const int nb = min(qb + 1, p.nb_row);
     for (int blk = lane; blk < nb; blk += 64)
       if (blk < p.init_blocks || blk > qb - p.local_blocks) row[blk] = INFINITY;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -703,15 +708,27 @@ static int run_cmp(CmpArgs& a) {
   if (a.what == 0) {
     cmp_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)(a.Hkv * a.p.GT)), 64 * (16 / FWD_TPW), 0, a.stream>>>(a.p);
   } else if (a.what == 1) {
-    const size_t dyn = (size_t)16 * a.sp.nb_cap * 4;
     // kernel 32 / stride 16 / block 64 (the published configuration) gets the compile-time fold
     const bool usual = a.sp.ks == 2 * a.sp.st && a.sp.bs == 4 * a.sp.st;
     const void* fn = usual ? (const void*)cmp_select_kernel<T, D, 2, 4> : (const void*)cmp_select_kernel<T, D, 0, 0>;
-    if (dyn > 64 * 1024) {
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess) return NSA_ERR_UNSUPPORTED;
+    // A workgroup's LDS is the K staging tiles plus 64 bytes per block a token of the tile can choose from.
+    // One launch sized for the longest sequence would leave a single workgroup per CU from ~1000 blocks
+    // on, so tiles are grouped by need: up to three launches, with row pitches for which three, two and
+    // one workgroup fit a CU's 160 KiB (workgroups of the other groups return at once).
+    const int tiles_bytes = 2 * 32 * lds_pitch(D) * (int)sizeof(T);
+    const int fits[3] = {(53760 - tiles_bytes) / 64, (80640 - tiles_bytes) / 64, 1 << 30};
+    int lo = 0;
+    for (int c = 0; c < 3 && lo < a.sp.nb_cap; c++) {
+      const int hi = a.sp.nb_cap < fits[c] ? a.sp.nb_cap : fits[c];
+      a.sp.nb_lo = lo; a.sp.nb_row = hi;
+      const size_t dyn = (size_t)16 * hi * 4;
+      if (dyn > 64 * 1024) {
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess) return NSA_ERR_UNSUPPORTED;
+      }
+      if (usual) cmp_select_kernel<T, D, 2, 4><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
+      else cmp_select_kernel<T, D, 0, 0><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
+      lo = hi;
     }
-    if (usual) cmp_select_kernel<T, D, 2, 4><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
-    else cmp_select_kernel<T, D, 0, 0><<<dim3((unsigned)slots, (unsigned)a.Hkv), 256, dyn, a.stream>>>(a.sp);
   } else {
     const CmpBwdLayout L = cmp_bwd_layout(a.Tq, a.Tk, a.B, a.Hq, a.Hkv, D);
     float* delta = (float*)(a.ws + L.delta);

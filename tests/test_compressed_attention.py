@@ -20,6 +20,7 @@ CASES = [
     ([900], 40, 2, 64, 64, 16, 128, 4, torch.float16),                 # G=20 (two head tiles), ks 64 / bs 128
     ([2100], 16, 1, 128, 32, 32, 64, 8, torch.bfloat16),               # non-overlapping windows (pad 0)
     ([17000], 4, 1, 32, 16, 16, 16, 6, torch.bfloat16),                # 1063 blocks: more than a lane keeps in registers
+    ([20000, 9000], 2, 1, 32, 16, 16, 16, 6, torch.bfloat16),          # 1250 blocks: the selection runs as three launches
 ]
 
 
