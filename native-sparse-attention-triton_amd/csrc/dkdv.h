@@ -24,7 +24,7 @@ static constexpr int MAX_CHUNK_TOKENS = 960;
 // `longest` is the size used by big launches (measured best: 768 for query lists, 960 for query ranges).
 static inline int dkdv_chunk_tokens(long long pairs, int longest) {
   if (pairs >= 2048ll * 1024) return longest < MAX_CHUNK_TOKENS ? longest : MAX_CHUNK_TOKENS;
-  if (pairs >= 2048ll * 512) return 512;
+  if (pairs >= 256ll * 1024) return 384;
   return 256;
 }
 
