@@ -27,7 +27,7 @@ HQ, HKV, D, BS = 64, 4, 128, 64
 H100_FWD_BWD_MS = 12.417 + 15.154
 # memory-side traffic per launch at the default workload (N=32768, top16), bytes: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, scaled by what the same counters read for a plain 1 GiB copy (x2.0 and x1.0); see profiles/
-MEASURED_TRAFFIC = {"fwd_attend": 15.9 * 2**30, "bwd_dq": 17.0 * 2**30, "bwd_dkdv": 18.1 * 2**30}
+MEASURED_TRAFFIC = {"fwd_attend": 15.8 * 2**30, "bwd_dq": 17.0 * 2**30, "bwd_dkdv": 18.3 * 2**30}
 
 
 def _events_ms(fn, iters):
