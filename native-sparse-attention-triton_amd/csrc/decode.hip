@@ -10,6 +10,7 @@
 // selected-block and the sliding-window branch share one partial launch, and one launch does both merges and
 // the gated sum with the compressed branch; the compressed branch's merge runs inside its block-selection kernel.
 #include "nsa_common.h"
+#include <type_traits>
 
 struct DecodeParams {
   const void* q; const void* k; const void* v; const int32_t* lens; const int32_t* idx;
@@ -257,7 +258,7 @@ static constexpr int MAX_SCORE_BLOCKS = 8192, MAX_SCORE_GROUP = 128;
 
 // One workgroup of SEL_NT threads per (kv-head, sequence): the work is a chain of short dependent phases, so
 // the aim is few round trips to memory and few barriers, not throughput.
-static constexpr int SEL_NT = 1024, SEL_NW = SEL_NT / 64, SEL_LDS_SCORES = 8192;
+static constexpr int SEL_NT = 1024, SEL_NW = SEL_NT / 64, SEL_LDS_SCORES = 8192, SEL_REG_BLOCKS = 16;
 
 template <typename T, int D>
 __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams p) {
@@ -365,30 +366,72 @@ __global__ __launch_bounds__(SEL_NT) void decode_score_select_kernel(ScoreParams
     if (blk < p.init_blocks || (blk <= qb && blk > qb - p.local_blocks)) v = INFINITY;
     bscore[blk] = v;
   }
-  // phase C: k_out rounds of (largest value, smallest index).  A thread only ever reads the entries it wrote
-  // in phase B (blk = tid mod SEL_NT), and it is the owner that retires a winner, so no barrier is needed
-  // around bscore; the wave maxima alternate between two LDS rows, which leaves one barrier per round.  Waves
-  // that own no block leave first (a barrier only counts the waves that are still alive), so with up to 64
-  // blocks a round is a single wave's lane exchanges.
-  const int nwc = min(SEL_NW, (p.max_blocks + 63) / 64);
-  if (wave >= nwc) return;
-  for (int round = 0; round < p.k_out; round++) {
-    float bv = -1.f;
-    int bi = 0x7fffffff;
-    for (int blk = tid; blk < p.max_blocks; blk += SEL_NT) {
-      const float v = bscore[blk];
-      if (v > bv) { bv = v; bi = blk; }
-    }
-    long long m = wave_max_i64(candidate_key(bv, bi));
-    if (nwc > 1) {
-      if (lane == 0) wave_best[round & 1][wave] = m;
+  // phase C: k_out rounds of (largest value, smallest index).
+  if (p.max_blocks <= 64 * SEL_REG_BLOCKS) {
+    // up to 1024 blocks: one wave keeps every candidate in registers (lane l owns blocks l, l + 64, ...), so a
+    // round is that wave's lane exchanges and nothing else - no LDS traffic, no barrier; the ids then leave
+    // in ascending order straight from the registers (ballot + prefix count per 64 blocks)
+    __syncthreads();
+    if (wave != 0) return;
+    int32_t* out = p.out_idx + (long long)h * p.osh + (long long)b * p.osb;
+    auto pick = [&](auto nreg_c) __attribute__((always_inline)) {
+      constexpr int NREG = decltype(nreg_c)::value;
+      float cand[NREG];
+#pragma unroll
+      for (int i = 0; i < NREG; i++) cand[i] = lane + 64 * i < p.max_blocks ? bscore[lane + 64 * i] : -3.f;
+      float bv = -1.f;
+      int bi = 0x7fffffff;
+#pragma unroll
+      for (int i = 0; i < NREG; i++)
+        if (cand[i] > bv) { bv = cand[i]; bi = lane + 64 * i; }
+      for (int round = 0; round < p.k_out; round++) {
+        const int win = candidate_index(wave_max_i64(candidate_key(bv, bi)));
+        if (bi == win) {
+          bv = -1.f; bi = 0x7fffffff;
+#pragma unroll
+          for (int i = 0; i < NREG; i++) {
+            if (lane + 64 * i == win) cand[i] = -2.f;
+            if (cand[i] > bv) { bv = cand[i]; bi = lane + 64 * i; }
+          }
+        }
+      }
+      // winners beyond the query's own block (possible only when fewer than k_out blocks are causal) sort
+      // last and are written as -1
+      int base = 0;
+#pragma unroll
+      for (int i = 0; i < NREG; i++) {
+        const int blk = lane + 64 * i;
+        const bool taken = cand[i] == -2.f && blk <= qb;
+        const unsigned long long mask = __ballot(taken);
+        if (taken) out[(long long)(base + __popcll(mask & ((1ull << lane) - 1ull))) * p.osk] = blk;
+        base += __popcll(mask);
+      }
+      for (int i = base + lane; i < p.k_out; i += 64) out[(long long)i * p.osk] = -1;
+    };
+    if (p.max_blocks <= 128) pick(std::integral_constant<int, 2>{});
+    else if (p.max_blocks <= 256) pick(std::integral_constant<int, 4>{});
+    else pick(std::integral_constant<int, SEL_REG_BLOCKS>{});
+    return;
+  } else {
+    // A thread only ever reads the entries it wrote in phase B (blk = tid mod SEL_NT), and it is the owner
+    // that retires a winner, so no barrier is needed around bscore; the wave maxima alternate between two
+    // LDS rows, which leaves one barrier per round.
+    for (int round = 0; round < p.k_out; round++) {
+      float bv = -1.f;
+      int bi = 0x7fffffff;
+      for (int blk = tid; blk < p.max_blocks; blk += SEL_NT) {
+        const float v = bscore[blk];
+        if (v > bv) { bv = v; bi = blk; }
+      }
+      const long long mine = wave_max_i64(candidate_key(bv, bi));
+      if (lane == 0) wave_best[round & 1][wave] = mine;
       __syncthreads();
-      m = wave_best[round & 1][0];
-      for (int w = 1; w < nwc; w++) { const long long o = wave_best[round & 1][w]; m = o > m ? o : m; }
+      long long m = wave_best[round & 1][0];
+      for (int w = 1; w < SEL_NW; w++) { const long long o = wave_best[round & 1][w]; m = o > m ? o : m; }
+      const int win = candidate_index(m);
+      if (tid == 0) picked[round] = win;
+      if ((win % SEL_NT) == tid) bscore[win] = -2.f;
     }
-    const int win = candidate_index(m);
-    if (tid == 0) picked[round] = win;
-    if ((win % SEL_NT) == tid) bscore[win] = -2.f;
   }
   // ascending order, ids beyond the query's block become -1 at the tail
   if (tid == 0) {
