@@ -678,8 +678,6 @@ struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, parti
 static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
   CmpBwdLayout L;
   L.max_blocks = Tk / 64 + B;
-  const int64_t GT = (Hq / Hkv + 15) / 16;
-  (void)GT;
   // queries per work item from a bound on the (query, key block) pairs (a causal range covers about half of Tq);
   // every block's range is at most Tq tokens: ceil(Tq/chunk)+1 items per segment is a safe bound
   L.chunk = dkdv_chunk_tokens(Hkv * L.max_blocks * Tq / 2, MAX_CHUNK_TOKENS);

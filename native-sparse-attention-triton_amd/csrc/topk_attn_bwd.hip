@@ -34,10 +34,8 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   BwdLayout L;
   L.max_blocks = T / bs + B;  // every sequence adds at most one ragged block
   L.n_pairs = Hkv * T * topk;
-  const int64_t GT = (Hq / Hkv + 15) / 16;
   const int chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
   L.max_items = (L.n_pairs + chunk - 1) / chunk + Hkv * L.max_blocks;
-  (void)GT;
   size_t tmp = 0;
   uint32_t* nk = nullptr;
   int32_t* nv = nullptr;
