@@ -152,16 +152,6 @@ __global__ __launch_bounds__(256) void decode_partial_pair_kernel(DecodeParams p
   else decode_partial_body<T, D, 0>(pb, blockIdx.x - blocks_a, v_s);
 }
 
-// Sum / maximum over the 64 lanes of a wave, returned to every lane, in a fixed order.
-__device__ __forceinline__ float wave_sum_f32(float x) {
-  x += dpp_f32<0xB1>(x); x += dpp_f32<0x4E>(x); x += dpp_f32<0x141>(x); x += dpp_f32<0x140>(x);
-  return column_sum(x);
-}
-__device__ __forceinline__ float wave_max_f32(float x) {
-  x = fmaxf(x, dpp_f32<0xB1>(x)); x = fmaxf(x, dpp_f32<0x4E>(x)); x = fmaxf(x, dpp_f32<0x141>(x)); x = fmaxf(x, dpp_f32<0x140>(x));
-  return column_max(x);
-}
-
 struct MergeScratch { float red_m[2], red_l[2]; float w_s[256]; };
 
 // Merged output column d = tid of one (sequence, query head): sum_c w_c O_c[d] / sum_c w_c l_c; m_out / l_out

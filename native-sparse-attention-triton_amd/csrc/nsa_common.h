@@ -137,6 +137,16 @@ template <int CTRL> __device__ __forceinline__ float dpp_f32(float x) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
 }
 
+// Sum / maximum over the 64 lanes of a wave, returned to every lane, in a fixed order.
+__device__ __forceinline__ float wave_sum_f32(float x) {
+  x += dpp_f32<0xB1>(x); x += dpp_f32<0x4E>(x); x += dpp_f32<0x141>(x); x += dpp_f32<0x140>(x);
+  return column_sum(x);
+}
+__device__ __forceinline__ float wave_max_f32(float x) {
+  x = fmaxf(x, dpp_f32<0xB1>(x)); x = fmaxf(x, dpp_f32<0x4E>(x)); x = fmaxf(x, dpp_f32<0x141>(x)); x = fmaxf(x, dpp_f32<0x140>(x));
+  return column_max(x);
+}
+
 // Wave-wide maximum of a signed 64-bit key, returned to every lane: four DPP steps inside each row of
 // 16 lanes (pair, quad, half-row mirror, row mirror), then the two lane swaps across rows.
 template <int CTRL> __device__ __forceinline__ long long dpp_exchange64(long long k) {

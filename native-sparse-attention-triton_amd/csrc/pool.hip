@@ -84,14 +84,14 @@ __global__ __launch_bounds__(256) void pool_dx_kernel(PoolParams p, const T* __r
 }
 
 // partial[h][tile][k]: one workgroup per (tile of DW_TILE output tokens, head)
-static constexpr int DW_TILE = 64;
+static constexpr int DW_TILE = 16;  // windows per workgroup of the dW pass: short tiles so that a few thousand windows still fill the chip
 template <typename T, int D>
 __global__ __launch_bounds__(256) void pool_dw_partial_kernel(PoolParams p, const T* __restrict__ dy, long long dysn, long long dysh,
                                                               float* __restrict__ partial, int n_tiles) {
   using v8 = typename Elem<T>::v8;
   constexpr int C = D / 8;            // threads per token
   constexpr int TPW = 256 / C;        // tokens in flight per pass
-  __shared__ float red[256];
+  __shared__ float red[4 * 16];
   const int tile = blockIdx.x, h = blockIdx.y;
   const int c = threadIdx.x % C, tl = threadIdx.x / C;
   const int n0 = tile * DW_TILE, n1 = min(p.total_y, n0 + DW_TILE);
@@ -113,17 +113,18 @@ __global__ __launch_bounds__(256) void pool_dw_partial_kernel(PoolParams p, cons
         }
       }
     }
+    // sum over the workgroup: lanes of a wave by lane exchanges, then the four waves through LDS
+    // (fixed order, so the result does not depend on scheduling)
 #pragma unroll
     for (int k = 0; k < 16; k++) {
-      red[threadIdx.x] = acc[k];
-      __syncthreads();
-      for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
-        __syncthreads();
-      }
-      if (threadIdx.x == 0 && k0 + k < p.ks) partial[((long long)h * n_tiles + tile) * p.ks + k0 + k] = red[0];
-      __syncthreads();
+      const float v = wave_sum_f32(acc[k]);
+      if ((threadIdx.x & 63) == 0) red[(threadIdx.x >> 6) * 16 + k] = v;
     }
+    __syncthreads();
+    if (threadIdx.x < 16 && k0 + threadIdx.x < p.ks)
+      partial[((long long)h * n_tiles + tile) * p.ks + k0 + threadIdx.x] =
+          ((red[threadIdx.x] + red[16 + threadIdx.x]) + red[32 + threadIdx.x]) + red[48 + threadIdx.x];
+    __syncthreads();
   }
 }
 
