@@ -300,6 +300,15 @@ int nsa_decode_branches_gate(const void* q, const void* sparse_k, const void* sp
 int nsa_gate_combine(const void* gate, const void* branch0, const void* branch1, const void* branch2, void* out, int64_t n_rows,
                      int64_t num_q_heads, int64_t head_dim, const int64_t* strides, int dtype, void* stream);
 
+/* Backward of the gated sum as autograd derives it from native_sparse_attention/module/native_sparse_attention.py:228-232:
+ * dbranch_i = gate[..., i] * dout, dgate[n, h, i] = sum over head_dim of dout * branch_i (products rounded to the
+ * element type, fp32 sum).  dgate [n_rows, Hq, 3] and the three dbranch [n_rows, Hq, D] are written densely.
+ * strides (HOST int64[11]): gate (n, h, k), branch0 (n, h), branch1 (n, h), branch2 (n, h), dout (n, h).
+ */
+int nsa_gate_combine_bwd(const void* gate, const void* branch0, const void* branch1, const void* branch2, const void* dout,
+                         void* dgate, void* dbranch0, void* dbranch1, void* dbranch2, int64_t n_rows, int64_t num_q_heads,
+                         int64_t head_dim, const int64_t* strides, int dtype, void* stream);
+
 /* ---- decode (one query per sequence over KV-cache slabs [B, slab_len, Hkv, D]) ---------------
  * strides: HOST int64 array: q(b,h) k(b,n,h) v(b,n,h) o(b,h) [+ idx(h,b,k) for the entry points
  * that read or write topk ids] = 10 or 13 values.  q/k/v strides must be multiples of 8.

@@ -654,23 +654,30 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
 // ------------------------------------------------------------------------------------------
 // dK/dV segments: blocks of 64 compressed keys per (head, sequence); their queries are the
 // contiguous range from the first position that sees the block's first key to the sequence end
-__global__ void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cu_k, int batch, int Hkv, int ks, int st,
-                                    int window, int max_blocks, int32_t* __restrict__ cu_blk, int32_t* __restrict__ seg_begin, int32_t* __restrict__ seg_end) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  int acc = 0;
-  cu_blk[0] = 0;
-  for (int b = 0; b < batch; b++) { acc += (cu_k[b + 1] - cu_k[b] + 63) / 64; cu_blk[b + 1] = acc; }
-  for (int h = 0; h < Hkv; h++) {
-    for (int g = 0; g < max_blocks; g++) { seg_begin[h * max_blocks + g] = 0; seg_end[h * max_blocks + g] = 0; }
-    for (int b = 0; b < batch; b++) {
+__global__ __launch_bounds__(256) void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cu_k, int batch, int Hkv, int ks, int st,
+                                                            int window, int max_blocks, int32_t* __restrict__ cu_blk, int32_t* __restrict__ seg_begin, int32_t* __restrict__ seg_end) {
+  // one workgroup: the prefix sum of the blocks per sequence goes through LDS (thread 0; batches are short
+  // lists), the Hkv * max_blocks segments are then filled by all threads
+  extern __shared__ int32_t blk_s[];  // [batch + 1]
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    blk_s[0] = 0; cu_blk[0] = 0;
+    for (int b = 0; b < batch; b++) { acc += (cu_k[b + 1] - cu_k[b] + 63) / 64; blk_s[b + 1] = acc; cu_blk[b + 1] = acc; }
+  }
+  __syncthreads();
+  const int n_blk = blk_s[batch];
+  for (int i = threadIdx.x; i < Hkv * max_blocks; i += 256) {
+    const int g = i % max_blocks;
+    int lo = 0, hi = 0;
+    if (g < n_blk) {
+      const int b = find_sequence(blk_s, batch, g);
       const int lq = cu_q[b + 1] - cu_q[b];
-      for (int g = cu_blk[b]; g < cu_blk[b + 1]; g++) {
-        const int first_pos = window == -2 ? 0 : (g - cu_blk[b]) * 64 * st + ks - 1;
-        seg_begin[h * max_blocks + g] = cu_q[b] + min(first_pos, lq);
-        // window mode (ordinary keys): the block's last key 64*g' + 63 is seen up to position 64*g' + 63 + window
-        seg_end[h * max_blocks + g] = cu_q[b] + (window < 0 ? lq : (int)min((long long)lq, (long long)(g - cu_blk[b]) * 64 + 64 + window));  // -1, -2: to the end
-      }
+      const int first_pos = window == -2 ? 0 : (g - blk_s[b]) * 64 * st + ks - 1;
+      lo = cu_q[b] + min(first_pos, lq);
+      // window mode (ordinary keys): the block's last key 64*g' + 63 is seen up to position 64*g' + 63 + window
+      hi = cu_q[b] + (window < 0 ? lq : (int)min((long long)lq, (long long)(g - blk_s[b]) * 64 + 64 + window));  // -1, -2: to the end
     }
+    seg_begin[i] = lo; seg_end[i] = hi;
   }
 }
 
@@ -738,7 +745,7 @@ static int run_cmp(CmpArgs& a) {
     // dQ first: it forms delta = rowsum(O * dO) from the dO rows it holds and leaves it behind for the dK/dV pass
     a.p.o = const_cast<void*>(a.o_in); a.p.delta = nullptr; a.p.delta_out = delta;
     cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
-    cmp_segments_kernel<<<1, 64, 0, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
+    cmp_segments_kernel<<<1, 256, (size_t)(a.B + 1) * 4, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
     chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off, L.chunk);
     DkdvParams d;
     d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;

@@ -45,6 +45,7 @@ _SIGNATURES = {
     "nsa_cache_stage_token": (c_int, [P] * 4 + [I] * 10 + [P]),
     "nsa_cache_commit_token": (c_int, [P] * 9 + [I] * 8 + [P]),
     "nsa_gate_combine": (c_int, [P] * 5 + [I] * 3 + [P, c_int, P]),
+    "nsa_gate_combine_bwd": (c_int, [P] * 9 + [I] * 3 + [P, c_int, P]),
     "nsa_decode_branches_gate_workspace_bytes": (Z, [I] * 7),
     "nsa_decode_branches_gate": (c_int, [P] * 13 + [I] * 8 + [P, F, c_int, P, Z, P]),
     "nsa_decode_prepare": (c_int, [P] * 8 + [F] + [P] * 8 + [I] * 4 + [P] + [I] * 6 + [c_int, P]),

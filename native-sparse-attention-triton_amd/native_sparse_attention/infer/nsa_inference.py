@@ -22,6 +22,7 @@ from ..ops import (
     weightedpool_compress,
 )
 from ..ops.decode import decode_branches_gate
+from ..ops.gated_sum import gate_combine
 from ..ops.sliding_window import sliding_window_attention_varlen
 from ..ops.utils import get_compressed_seqlens, last_dim_contiguous
 
@@ -90,21 +91,6 @@ def sliding_window_attention_infer(cu_seqlens, step, query, key, value, cache, w
     # the ring holds min(tokens seen, window_size) rows; the kernel clips the count to the slab by itself
     return flash_attention_decode(query, cache.sliding_kv_cache[0, :batch], cache.sliding_kv_cache[1, :batch],
                                   cache.sliding_kv_len[:batch])
-
-
-def gate_combine(gate_value, branch0, branch1, branch2):
-    """gate_value[..., 0, None] * branch0 + gate_value[..., 1, None] * branch1 + gate_value[..., 2, None] * branch2
-    (nsa_inference.py:146-150 of the reference) in one kernel, bit-identical to that expression.  No autograd."""
-    assert gate_value.shape == branch0.shape[:2] + (3,) and branch0.shape == branch1.shape == branch2.shape
-    assert gate_value.dtype == branch0.dtype == branch1.dtype == branch2.dtype
-    a, b, c = (last_dim_contiguous(t) for t in (branch0, branch1, branch2))
-    out = torch.empty_like(a, memory_format=torch.contiguous_format)
-    strides = _lib.host_i64([gate_value.stride(0), gate_value.stride(1), gate_value.stride(2), a.stride(0), a.stride(1), b.stride(0),
-                             b.stride(1), c.stride(0), c.stride(1), out.stride(0), out.stride(1)])
-    rc = _lib.load().nsa_gate_combine(gate_value.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), out.data_ptr(), a.shape[0],
-                                      a.shape[1], a.shape[2], strides, _lib.dtype_code(a), _lib.stream_ptr(a))
-    _lib.check(rc, "nsa_gate_combine")
-    return out
 
 
 def nsa_infer(

@@ -10,6 +10,7 @@ import torch
 
 from ..infer import nsa_infer
 from ..ops import avgpool_compress, compressed_attention, linear_compress, topk_sparse_attention, weightedpool_compress
+from ..ops.gated_sum import gated_sum
 from ..ops.sliding_window import sliding_window_attention_varlen
 from .kv_cache import NSACache
 from .rope import RopeConfig, RotaryEmbedding
@@ -99,8 +100,8 @@ class NativeSparseAttention(torch.nn.Module):
         sliding_attn_output = sliding_window_attention_varlen(q, k, v, cu_seqlens, self.window_size)
 
         gate = self.gate(x).view(-1, self.num_q_heads, 3)
-        attn_output = (gate[..., 0:1] * compressed_attn_output + gate[..., 1:2] * sparse_attn_output
-                       + gate[..., 2:3] * sliding_attn_output)
+        # gate[..., 0:1] * compressed + gate[..., 1:2] * sparse + gate[..., 2:3] * sliding (:228-232), one kernel each way
+        attn_output = gated_sum(gate, compressed_attn_output, sparse_attn_output, sliding_attn_output)
         return self.proj_o(attn_output.reshape(-1, self.num_q_heads * self.head_dim))
 
     @torch.no_grad()
