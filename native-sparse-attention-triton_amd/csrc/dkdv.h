@@ -1,15 +1,16 @@
 // dK/dV pass shared by the block-sparse and the compressed attention backward.
 //
 // A workgroup keeps one block of BS keys (K and V rows) in registers, each wave 16*KT of them as
-// MFMA B operands, and streams query rows through double-buffered LDS two (token, head-tile) row
-// groups at a time.  P and dS leave the score MFMA already in B-operand layout; the transposed
+// MFMA B operands, and streams query rows two (token, head-tile) row groups at a time through three
+// LDS buffers that asynchronous global-to-LDS copies fill two steps ahead.  P and dS leave the score MFMA already in B-operand layout; the transposed
 // Q and dO fragments are read from LDS with ds_read_b64_tr_b16.  Work items are (segment,
 // chunk of up to MAX_CHUNK_TOKENS queries); each writes an fp32 partial, a second kernel adds the chunks of
 // a segment in order, so no atomics are needed and results are reproducible.
 //   RANGE = false: the queries of a segment come from a sorted list (reverse index of topk_idx),
 //                  key j is visible to a query at position pos iff j <= pos.
-//   RANGE = true : the queries are the contiguous range [seg_off[s], seg_off[s+1]) of global token
-//                  ids, keys are compressed tokens: visible iff j*st + ks - 1 <= pos.
+//   RANGE = true : the queries are the contiguous range [seg_begin[s], seg_end[s]) of global token ids;
+//                  DkdvParams::window says which keys a position sees (compressed keys, a sliding
+//                  window of ordinary keys, or all of them).
 #pragma once
 #include "nsa_common.h"
 
