@@ -1,10 +1,10 @@
 // Attention of queries over compressed keys/values (compressed_attention), forward, block
 // selection and backward.
 //
-// Tiling: a workgroup owns 16 consecutive query tokens of one sequence and one kv-head (each of
-// its 4 waves 4 tokens x the <=16 query heads of the GQA group); compressed K/V chunks of 32 keys
-// are staged once per workgroup in double-buffered LDS and shared by the 16 tokens, which see
-// almost the same causal range (key c is visible to position i iff c*stride + kernel - 1 <= i).
+// Tiling: a workgroup owns 16 (forward, selection) or 8 (dQ) consecutive query tokens of one
+// sequence and one kv-head, each wave 2 or 4 tokens x the <=16 query heads of the GQA group;
+// compressed K/V chunks of 32 keys are staged once per workgroup in double-buffered LDS and
+// shared by those tokens, which see almost the same causal range (key c is visible to position i iff c*stride + kernel - 1 <= i).
 // Scores are produced transposed (S^T = K Q^T) so that one lane holds one head and P^T / dS^T
 // feed the next MFMA directly; V^T and K^T fragments are read from the row-major LDS tiles with
 // ds_read_b64_tr_b16.

@@ -1,15 +1,17 @@
 // Backward of block-sparse GQA attention (topk_sparse_attention): dQ, dK, dV.
 //
-// Passes, all on the caller's stream and out of the caller's workspace:
-//   1. delta[h][t] = sum_d O*dO.
-//   2. Reverse index "KV block -> queries that selected it": one (key = head*blocks + block,
+// Passes, all on the caller's stream and out of the caller's workspace (run in the order 1, 3, 2: the dQ
+// pass leaves delta behind for the dK/dV pass):
+//   1. Reverse index "KV block -> queries that selected it": one (key = head*blocks + block,
 //      value = token) pair per valid topk_idx entry, stable radix sort by key (tokens stay
 //      ascending inside a block), segment offsets by binary search.  No host round trips.
-//   3. dK/dV: a workgroup keeps one KV block's K and V rows in registers (each wave owns 16
+//   2. dK/dV: a workgroup keeps one KV block's K and V rows in registers (each wave owns 16
 //      keys) and streams the queries of that block two tokens at a time through LDS; per-chunk
 //      fp32 partials are reduced in a fixed order, so the result is deterministic (no atomics).
-//   4. dQ: one wavefront per (token, kv-head), same dataflow as the forward kernel; the K rows are
-//      written through to wave-private LDS and read back transposed for dQ^T += K^T * dS^T.
+//   3. dQ: one wavefront per (token, kv-head), same dataflow as the forward kernel; the K rows are
+//      written through to wave-private LDS and read back transposed for dQ^T += K^T * dS^T.  It
+//      also forms delta[h][t] = sum_d O*dO from the dO rows it holds (a delta pass of its own
+//      runs only when the index phase is requested alone).
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
