@@ -85,7 +85,12 @@ class NativeSparseAttention(torch.nn.Module):
         # keys and values are compressed before the rotary embedding (:172-188)
         compressed_k, compressed_cu_seqlens = self.compress_func(k, self.compress_key, cu_seqlens, self.kernel_size, self.kernel_stride,
                                                                  self.intra_block_pe)
-        compressed_v, _ = self.compress_func(v, self.compress_value, cu_seqlens, self.kernel_size, self.kernel_stride, None)
+        # the values compress to the same rows as the keys: no second device read for the output shape
+        if self.compress_func in (avgpool_compress, weightedpool_compress, linear_compress):
+            compressed_v, _ = self.compress_func(v, self.compress_value, cu_seqlens, self.kernel_size, self.kernel_stride, None,
+                                                 known_total=compressed_k.shape[0], known_y_cu=compressed_cu_seqlens)
+        else:
+            compressed_v, _ = self.compress_func(v, self.compress_value, cu_seqlens, self.kernel_size, self.kernel_stride, None)
 
         q = self.rope(q, cu_seqlens)
         compressed_k = self.rope(compressed_k, compressed_cu_seqlens, stride=self.kernel_stride)
