@@ -1,6 +1,7 @@
 """Seeded sweep over ragged shapes, head layouts, head sizes, block sizes and dtypes: forward and backward of the
 block-sparse attention, the compressed attention with its block selection, and the sliding-window / dense causal
-attention against the oracle (or a masked softmax where the oracle has no such function)."""
+attention against the oracle (or a masked softmax where the oracle has no such function); the same for the decode
+operators."""
 import random
 
 import pytest
@@ -83,3 +84,51 @@ def test_random_shapes(device, seed):
         assert_close(o, want, "o")
         for name, a, b in (("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)):
             assert_close(a, b, name, rel_to=max(1.0, b.abs().max().item()))
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_decode_shapes(device, seed):
+    """The three decode operators against the oracle, and the fused selected + window branches + gated sum against
+    the separate calls (bit for bit), on random batches, slab sizes, head layouts and block sizes."""
+    from native_sparse_attention.ops import compressed_attention_decode, flash_attention_decode, topk_sparse_attention_decode
+    from native_sparse_attention.ops.decode import decode_branches_gate
+    from native_sparse_attention.ops.gated_sum import gate_combine
+
+    rng = random.Random(2000 + seed)
+    for case in range(10):
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        d, Hkv, G = rng.choice([32, 64, 96, 128]), rng.choice([1, 2, 3]), rng.choice([1, 2, 4, 8, 16, 20])
+        Hq = Hkv * G
+        B, bs, topk = rng.randint(1, 6), rng.choice([32, 64, 128]), rng.randint(1, 8)
+        lens = [rng.choice([1, 2, 31, 33, 64, 65, 127, 129, 500, 1000, 2049]) for _ in range(B)]
+        slab = max(lens) + rng.randint(0, 70)
+        print("case", seed, case, lens, Hq, Hkv, d, bs, topk, dtype, flush=True)
+        g = torch.Generator(device=device).manual_seed(100 * seed + case)
+        q = torch.randn(B, Hq, d, generator=g, device=device).to(dtype)
+        cache = torch.randn(2, B + 1, slab, Hkv, d, generator=g, device=device).to(dtype)   # slabs are views, as in a cache
+        k, v = cache[0, :B], cache[1, :B]
+        seqlens = torch.tensor(lens, dtype=torch.int32, device=device)
+        o_dense = flash_attention_decode(q, k, v, seqlens)
+        assert_close(o_dense, oracle.dense_attention_decode(q.float(), k.float(), v.float(), seqlens), "dense o")
+        idx = torch.stack([make_topk_idx(cu_from_lens([L], device), bs, topk, Hkv, seed=7 * case + b)[:, L - 1]
+                           for b, L in enumerate(lens)], 1).contiguous()
+        o_sel = topk_sparse_attention_decode(q, k, v, idx, bs, seqlens)
+        assert_close(o_sel, oracle.topk_sparse_attention_decode(q.float(), k.float(), v.float(), idx, bs, seqlens), "topk o")
+        ks, st = rng.choice([(32, 16), (16, 16), (64, 16)])
+        cbs = rng.choice([x for x in (64, 128) if x % ks == 0])
+        clens = torch.tensor([0 if L < ks else (L - ks) // st + 1 for L in lens], dtype=torch.int32, device=device)
+        cslab = max(int(clens.max()), 1) + rng.randint(0, 5)
+        ck, cv = cache[0, :B, :cslab], cache[1, :B, :cslab]
+        k_sel = rng.randint(1, 8)
+        o_cmp, sel = compressed_attention_decode(q, ck, cv, seqlens, clens, ks, st, cbs, k_sel)
+        want_cmp, want_sel = oracle.compressed_attention_decode(q.float(), ck.float(), cv.float(), seqlens, clens, ks, st, cbs, k_sel)
+        assert_close(o_cmp, want_cmp, "cmp o")
+        assert sel.shape == want_sel.shape and (sel != want_sel).any(-1).float().mean().item() <= 0.1
+        W = min(slab, rng.choice([16, 64, 512]))
+        wk, wv = cache[0, 1:B + 1, :W], cache[1, 1:B + 1, :W]
+        wlen = torch.tensor([min(L, W) for L in lens], dtype=torch.int32, device=device)
+        gate = torch.sigmoid(torch.randn(B, Hq, 3, generator=g, device=device)).to(dtype)
+        out, f_sel, f_win = decode_branches_gate(q, k, v, seqlens, idx, bs, wk, wv, wlen, o_cmp, gate)
+        o_win = flash_attention_decode(q, wk, wv, wlen)
+        assert torch.equal(f_sel, o_sel) and torch.equal(f_win, o_win)
+        assert torch.equal(out, gate_combine(gate, o_cmp, o_sel, o_win))
