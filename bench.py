@@ -257,6 +257,45 @@ def bench_decode(args, dev):
     }
 
 
+def bench_layer(args, dev):
+    """Layer benchmark of the reference's test/test_nsa_module.py:20-60,103-150: NativeSparseAttention against the dense
+    SelfAttention layer, hidden 8192, 64q/4kv heads, d=128, one sequence of --seqlen tokens; forward (no grad) and
+    forward + backward.  The projections are rocBLAS GEMMs (plumbing); everything else runs on this library's kernels."""
+    from native_sparse_attention.module import NativeSparseAttention, RopeConfig, SelfAttention
+
+    rope = RopeConfig(max_position_embeddings=131072, head_dim=D, rope_theta=500000,
+                      rope_scaling={"factor": 8.0, "high_freq_factor": 4.0, "low_freq_factor": 1.0,
+                                    "original_max_position_embeddings": 8192, "rope_type": "llama3"})
+    torch.manual_seed(42)
+    nsa = NativeSparseAttention(compress_type="avgpool", hidden_size=8192, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D,
+                                kernel_size=32, kernel_stride=16, block_size=BS, topk=16, init_blocks=1, local_blocks=2,
+                                window_size=512, rope_config=rope).to(dev).to(torch.bfloat16)
+    dense = SelfAttention(hidden_size=8192, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D, rope_config=rope).to(dev).to(torch.bfloat16)
+    N = args.seqlen
+    x = torch.randn(N, 8192, device=dev, dtype=torch.bfloat16)
+    cu = torch.tensor([0, N], device=dev, dtype=torch.int32)
+    xg = x.clone().requires_grad_()
+    it = max(2, min(args.steps, 5))
+
+    def fwd_bwd(layer):
+        y = layer(xg, cu)
+        (y * y).sum().backward()
+    with torch.no_grad():
+        t_nsa_f = _time_ms(lambda: nsa(x, cu), it)
+        t_dense_f = _time_ms(lambda: dense(x, cu), it)
+    t_nsa = _time_ms(lambda: fwd_bwd(nsa), it)
+    t_dense = _time_ms(lambda: fwd_bwd(dense), it)
+    return {
+        "metric": "NSA attention layer forward+backward ms (hidden 8192, N=%d)" % N, "value": t_nsa, "unit": "ms", "n_gpus": 1,
+        "steps": it, "warmup": 2, "ms_per_step": t_nsa, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "NativeSparseAttention layer, hidden 8192, 64q/4kv heads, d=128, avgpool kernel 32 stride 16, block 64, "
+                               "top-16, window 512, one sequence of %d tokens" % N,
+                   "ms": {"nsa_forward": t_nsa_f, "nsa_forward_backward": t_nsa, "dense_self_attention_forward": t_dense_f,
+                          "dense_self_attention_forward_backward": t_dense}},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -269,8 +308,8 @@ def main():
                     help="also run three plain 1 GiB device copies (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--readme-heads", action="store_true",
                     help="compressed workload with the 64q/4kv head layout of the reference README tables instead of config 3's 32q/2kv")
-    ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode"],
-                    help="topk = the headline metric (default); the others time the pipeline, long-sequence compressed-attention and decode benchmarks")
+    ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode", "layer"],
+                    help="topk = the headline metric (default); the others time the pipeline, long-sequence compressed-attention, decode and whole-layer benchmarks")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the operator path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -283,7 +322,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload != "topk":
-        fn = {"pipeline": bench_pipeline, "compressed": bench_compressed, "decode": bench_decode}[args.workload]
+        fn = {"pipeline": bench_pipeline, "compressed": bench_compressed, "decode": bench_decode, "layer": bench_layer}[args.workload]
         print(json.dumps(fn(args, dev)))
         return
     N, topk = args.seqlen, args.topk
