@@ -93,3 +93,28 @@ def test_decode_step_entry_points_check_their_arguments():
     rc = lib.nsa_decode_branches_gate(fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, 4, 32, 2, 128, 8192, 512,
                                       8, 64, strides28, 0.088, 0, fake, need - 1, None)
     assert rc == -3
+
+
+def test_reference_import_paths_resolve():
+    """The names the reference's callers and scripts import (native_sparse_attention/ops/__init__.py:15-53,
+    infer/__init__.py:15, infer/nsa_inference.py:16-22, module/__init__.py, model/__init__.py, module/kv_cache.py:18)
+    exist under the same module paths; importing needs neither a GPU nor the shared library."""
+    import importlib
+
+    wanted = {
+        "native_sparse_attention.ops": ["avgpool_compress", "weightedpool_compress", "linear_compress", "flash_attention_varlen",
+                                        "compressed_attention", "topk_sparse_attention", "flash_attention_decode",
+                                        "compressed_attention_decode", "topk_sparse_attention_decode"],
+        "native_sparse_attention.ops.triton.utils": ["get_compressed_seqlens"],
+        "native_sparse_attention.ops.topk_sparse_attention": ["_topk_sparse_attention_fwd", "_topk_sparse_attention_bwd"],
+        "native_sparse_attention.ops.compressed_attention": ["_compressed_attention_bwd"],
+        "native_sparse_attention.infer": ["nsa_infer"],
+        "native_sparse_attention.infer.inference_func": ["compress_infer", "compressed_attention_infer", "topk_sparse_attention_infer",
+                                                         "sliding_window_attention_infer"],
+        "native_sparse_attention.module": ["NativeSparseAttention", "SelfAttention", "RopeConfig", "RotaryEmbedding", "NSACache", "KVCache"],
+        "native_sparse_attention.model": ["ToyNSALlama", "ToyNSALlamaConfig", "ToyLlama", "ToyLlamaConfig", "InferenceConfig"],
+    }
+    for module, names in wanted.items():
+        mod = importlib.import_module(module)
+        for name in names:
+            assert hasattr(mod, name), "%s.%s" % (module, name)
