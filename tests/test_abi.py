@@ -97,7 +97,8 @@ def test_decode_step_entry_points_check_their_arguments():
 
 def test_reference_import_paths_resolve():
     """The names the reference's callers and scripts import (native_sparse_attention/ops/__init__.py:15-53,
-    infer/__init__.py:15, infer/nsa_inference.py:16-22, module/__init__.py, model/__init__.py, module/kv_cache.py:18)
+    infer/__init__.py:15, infer/nsa_inference.py:16-22, module/__init__.py, model/__init__.py, module/kv_cache.py:18,
+    test/test_topk_sparse_attention.py:16-31)
     exist under the same module paths; importing needs neither a GPU nor the shared library."""
     import importlib
 
@@ -106,6 +107,15 @@ def test_reference_import_paths_resolve():
                                         "compressed_attention", "topk_sparse_attention", "flash_attention_decode",
                                         "compressed_attention_decode", "topk_sparse_attention_decode"],
         "native_sparse_attention.ops.triton.utils": ["get_compressed_seqlens"],
+        "native_sparse_attention.ops.triton.topk_sparse_attention": ["topk_sparse_attention", "_topk_sparse_attention_fwd",
+                                                                      "_topk_sparse_attention_bwd"],
+        "native_sparse_attention.ops.triton.compressed_attention": ["compressed_attention", "_compressed_attention_fwd",
+                                                                     "_compressed_attention_bwd"],
+        "native_sparse_attention.ops.triton.flash_attention": ["flash_attention_varlen", "_flash_attention_fwd", "_flash_attention_bwd"],
+        "native_sparse_attention.ops.triton.linear_compress": ["linear_compress"],
+        "native_sparse_attention.ops.triton.weighted_pool": ["weightedpool_compress", "avgpool_compress"],
+        "native_sparse_attention.ops.triton.flash_attention_decode": ["flash_attention_decode"],
+        "native_sparse_attention.ops.triton.topk_sparse_attention_decode": ["topk_sparse_attention_decode"],
         "native_sparse_attention.ops.topk_sparse_attention": ["_topk_sparse_attention_fwd", "_topk_sparse_attention_bwd"],
         "native_sparse_attention.ops.compressed_attention": ["_compressed_attention_bwd"],
         "native_sparse_attention.infer": ["nsa_infer"],
