@@ -65,6 +65,13 @@ def compute_inv_freq(config: RopeConfig, device=None):
     return torch.where(medium, smoothed, scaled), 1.0
 
 
+def rotate_half(x):
+    """(-x2, x1) for x = (x1, x2) split in the middle of the last dimension (rope.py:53-58 of the reference).  Kept for
+    callers that build the rotation from tensors; RotaryEmbedding.forward does not use it."""
+    half = x.shape[-1] // 2
+    return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+
 def _rope_launch(x, inv_freq, scaling, cu_seqlens, step, stride, inverse):
     x = last_dim_contiguous(x)
     out = torch.empty_like(x, memory_format=torch.contiguous_format)
@@ -123,6 +130,28 @@ class RotaryEmbedding(nn.Module):
         assert x.dim() == 3 and x.shape[-1] == self.config.head_dim and position_index.dtype == torch.int32
         assert position_index.shape[0] == x.shape[0] and position_index.is_contiguous()
         return _rope_launch(x, self._frequencies(), float(self.attention_scaling), position_index, -1, int(stride), False)
+
+    @torch.no_grad()
+    def generate_cos_sin(self, x, position_ids):
+        """cos / sin tables [len, D] in x's dtype for position_ids [1, len] (rope.py:120-155 of the reference, without its
+        class-level cache): angle = position * inv_freq in fp32, both halves of the last dimension alike, times the
+        attention scaling.  Not used by forward (the kernel forms the angles itself)."""
+        angles = position_ids.reshape(-1, 1).float() * self.inv_freq.float()[None, :]
+        cos = (angles.cos() * self.attention_scaling).to(x.dtype)
+        sin = (angles.sin() * self.attention_scaling).to(x.dtype)
+        return torch.cat([cos, cos], dim=-1), torch.cat([sin, sin], dim=-1)
+
+    @torch.no_grad()
+    def generate_pos_embs(self, x, cu_seqlens, seqlens, step=0, stride=1):
+        """Per-row cos / sin [N, D] as rope.py:157-197 of the reference: step == 0 gives row i of a sequence position
+        i * stride, step > 0 gives sequence b the single position (len_b + step - 1) * stride."""
+        if step == 0:
+            total = int(cu_seqlens[-1])
+            start = torch.repeat_interleave(cu_seqlens[:-1].long(), seqlens.long(), output_size=total)
+            position = (torch.arange(total, device=x.device) - start) * stride
+        else:
+            position = (seqlens.long() + step - 1) * stride
+        return self.generate_cos_sin(x, position[None, :])
 
     def forward(self, x, cu_seqlens, step=0, stride=1):
         assert x.dim() == 3 and x.shape[-1] == self.config.head_dim

@@ -110,3 +110,25 @@ def test_module_cast_to_bf16_rounds_the_frequencies_like_the_reference(device):
     want = _reference_forward(x, rope.inv_freq.float(), pos)
     assert torch.isfinite(y).all()
     assert ((y.float() - want.float()).abs() <= 2.0 ** -7 * want.float().abs().clamp(min=1.0)).all()
+
+
+def test_tensor_level_helpers_agree_with_the_closed_form():
+    """rotate_half / generate_cos_sin / generate_pos_embs (the reference's tensor-level helpers, rope.py:53-58,120-197):
+    x * cos + rotate_half(x) * sin built from them is the textbook rotation of each (x1, x2) pair by position * inv_freq
+    (checked in fp64 on the CPU), for prefill rows and for a decode step."""
+    from native_sparse_attention.module.rope import rotate_half
+
+    rope = RotaryEmbedding(RopeConfig(head_dim=16, rope_scaling=None, rope_theta=100.0), device="cpu")
+    cu = torch.tensor([0, 3, 8], dtype=torch.int32)
+    seqlens = cu[1:] - cu[:-1]
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(8, 2, 16, generator=g, dtype=torch.float64)
+    assert torch.equal(rotate_half(x), torch.cat((-x[..., 8:], x[..., :8]), -1))
+    for step, stride, rows, positions in ((0, 4, x, [0, 4, 8, 0, 4, 8, 12, 16]), (2, 1, x[:2], [4, 6])):
+        cos, sin = rope.generate_pos_embs(rows, cu, seqlens, step=step, stride=stride)
+        assert cos.shape == (rows.shape[0], 16) and cos.dtype == rows.dtype
+        got = rows * cos[:, None, :] + rotate_half(rows) * sin[:, None, :]
+        ang = torch.tensor(positions, dtype=torch.float64)[:, None] * rope.inv_freq.double()[None, :]
+        x1, x2 = rows[..., :8], rows[..., 8:]
+        want = torch.cat((x1 * ang.cos()[:, None] - x2 * ang.sin()[:, None], x2 * ang.cos()[:, None] + x1 * ang.sin()[:, None]), -1)
+        assert torch.allclose(got, want, atol=1e-6)
