@@ -128,14 +128,16 @@ __global__ __launch_bounds__(256) void pool_dw_partial_kernel(PoolParams p, cons
   }
 }
 
+// dw[h][k] = sum over the tiles' partials: one wave per (h, k); lane l adds tiles l, l + 64, ... in order, then
+// the lanes meet in a fixed-order wave sum (reproducible whatever the number of tiles).
 template <typename T>
-__global__ void pool_dw_final_kernel(const float* __restrict__ partial, int n_tiles, int H, int ks, T* __restrict__ dw, long long dwsh) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;  // (h, k)
-  if (i >= H * ks) return;
+__global__ __launch_bounds__(64) void pool_dw_final_kernel(const float* __restrict__ partial, int n_tiles, int H, int ks, T* __restrict__ dw, long long dwsh) {
+  const int i = blockIdx.x;  // (h, k)
   const int h = i / ks, k = i % ks;
   float acc = 0.f;
-  for (int t = 0; t < n_tiles; t++) acc += partial[((long long)h * n_tiles + t) * ks + k];
-  dw[(long long)h * dwsh + k] = (T)acc;
+  for (int t = threadIdx.x; t < n_tiles; t += 64) acc += partial[((long long)h * n_tiles + t) * ks + k];
+  acc = wave_sum_f32(acc);
+  if (threadIdx.x == 0) dw[(long long)h * dwsh + k] = (T)acc;
 }
 
 template <typename T, int D>
@@ -152,7 +154,7 @@ static int pool_bwd_t(const PoolParams& p, const void* dy, long long dysn, long 
   if (dw) {
     const int n_tiles = (p.total_y + DW_TILE - 1) / DW_TILE;
     if (n_tiles > 0) pool_dw_partial_kernel<T, D><<<dim3((unsigned)n_tiles, (unsigned)p.H), 256, 0, s>>>(p, (const T*)dy, dysn, dysh, partial, n_tiles);
-    pool_dw_final_kernel<T><<<(p.H * p.ks + 255) / 256, 256, 0, s>>>(partial, n_tiles, p.H, p.ks, (T*)dw, dwsh);
+    pool_dw_final_kernel<T><<<p.H * p.ks, 64, 0, s>>>(partial, n_tiles, p.H, p.ks, (T*)dw, dwsh);
   }
   return nsa_check_launch();
 }
