@@ -656,14 +656,11 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
 // contiguous range from the first position that sees the block's first key to the sequence end
 __global__ __launch_bounds__(256) void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cu_k, int batch, int Hkv, int ks, int st,
                                                             int window, int max_blocks, int32_t* __restrict__ cu_blk, int32_t* __restrict__ seg_begin, int32_t* __restrict__ seg_end) {
-  // one workgroup: the prefix sum of the blocks per sequence goes through LDS (thread 0; batches are short
-  // lists), the Hkv * max_blocks segments are then filled by all threads
+  // one workgroup: the prefix sum of the 64-key blocks per sequence first (kept in LDS as well, for the
+  // searches below), then the Hkv * max_blocks segments are filled by all threads
   extern __shared__ int32_t blk_s[];  // [batch + 1]
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    blk_s[0] = 0; cu_blk[0] = 0;
-    for (int b = 0; b < batch; b++) { acc += (cu_k[b + 1] - cu_k[b] + 63) / 64; blk_s[b + 1] = acc; cu_blk[b + 1] = acc; }
-  }
+  block_count_prefix_256(cu_k, batch, 64, cu_blk);
+  for (int b = threadIdx.x; b <= batch; b += 256) blk_s[b] = cu_blk[b];
   __syncthreads();
   const int n_blk = blk_s[batch];
   for (int i = threadIdx.x; i < Hkv * max_blocks; i += 256) {

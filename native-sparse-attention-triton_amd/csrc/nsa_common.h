@@ -185,6 +185,32 @@ __device__ __forceinline__ long long candidate_key(float score, int index) {
 }
 __device__ __forceinline__ int candidate_index(long long key) { return 0x7fffffff - (int)(unsigned)(unsigned long long)key; }
 
+// out[0] = 0, out[b + 1] = sum over sequences <= b of ceil((cu[b + 1] - cu[b]) / unit): the prefix sum of the number
+// of unit-sized blocks per sequence, by one workgroup of 256 threads (thread t owns a contiguous run of sequences,
+// the 256 run totals are scanned in LDS).  Every thread of the workgroup must call it; ends with a barrier.
+__device__ __forceinline__ void block_count_prefix_256(const int32_t* __restrict__ cu, int batch, int unit, int32_t* __restrict__ out) {
+  __shared__ int run_total[256];
+  const int tid = threadIdx.x, per = (batch + 255) / 256;
+  const int b0 = min(batch, tid * per), b1 = min(batch, b0 + per);
+  int sum = 0;
+  for (int b = b0; b < b1; b++) sum += (cu[b + 1] - cu[b] + unit - 1) / unit;
+  run_total[tid] = sum;
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {
+    const int v = tid >= d ? run_total[tid - d] : 0;
+    __syncthreads();
+    run_total[tid] += v;
+    __syncthreads();
+  }
+  int acc = run_total[tid] - sum;
+  if (tid == 0) out[0] = 0;
+  for (int b = b0; b < b1; b++) {
+    acc += (cu[b + 1] - cu[b] + unit - 1) / unit;
+    out[b + 1] = acc;
+  }
+  __syncthreads();
+}
+
 // Index of the sequence that holds global token t: largest b with cu[b] <= t.
 __device__ __forceinline__ int find_sequence(const int32_t* __restrict__ cu, int batch, int t) {
   int lo = 0, hi = batch;  // invariant: cu[lo] <= t < cu[hi]

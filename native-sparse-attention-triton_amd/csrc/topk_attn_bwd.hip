@@ -64,15 +64,8 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
 
 // ------------------------------------------------------------------------------------------
 // pass 2: reverse index
-__global__ void seq_blocks_kernel(const int32_t* __restrict__ cu, int batch, int bs, int32_t* __restrict__ cu_blk) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    int acc = 0;
-    cu_blk[0] = 0;
-    for (int b = 0; b < batch; b++) {
-      acc += (cu[b + 1] - cu[b] + bs - 1) / bs;
-      cu_blk[b + 1] = acc;
-    }
-  }
+__global__ __launch_bounds__(256) void seq_blocks_kernel(const int32_t* __restrict__ cu, int batch, int bs, int32_t* __restrict__ cu_blk) {
+  block_count_prefix_256(cu, batch, bs, cu_blk);
 }
 
 __global__ __launch_bounds__(256) void emit_pairs_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ cu,
@@ -282,7 +275,7 @@ static int build_reverse_index(const BwdArgs& a, const BwdLayout& L) {
   int32_t* seg_off = (int32_t*)(ws + L.seg_off);
   int32_t* chunk_off = (int32_t*)(ws + L.chunk_off);
   const int n_seg = (int)(a.Hkv * L.max_blocks);
-  seq_blocks_kernel<<<1, 64, 0, a.stream>>>(a.cu, (int)a.B, (int)a.bs, cu_blk);
+  seq_blocks_kernel<<<1, 256, 0, a.stream>>>(a.cu, (int)a.B, (int)a.bs, cu_blk);
   emit_pairs_kernel<<<(unsigned)((L.n_pairs + 255) / 256), 256, 0, a.stream>>>(
       a.idx, a.cu, cu_blk, (int)a.B, (int)a.T, (int)a.Hkv, (int)a.topk, (int)a.bs, (int)L.max_blocks, a.ish, a.isn, a.isk, keys_in, vals_in);
   unsigned bits = 1;

@@ -115,3 +115,35 @@ def test_window_and_dense_attention(device, lens):
         o.backward(do)
         want.backward(do.float())
         _grads_close((("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)))
+
+
+def test_many_short_sequences(device):
+    """300 sequences (more than one per thread of the 256-thread prefix sums over the batch), some of them empty:
+    block-sparse and compressed attention, forward and backward."""
+    import random
+    rng = random.Random(5)
+    lens = [rng.choice([0, 1, 17, 33, 64, 65, 100, 130]) for _ in range(300)]
+    print("case", len(lens), sum(lens), flush=True)
+    cu, q, k, v, do, g = _tensors(lens, device)
+    idx = make_topk_idx(cu, BS, TOPK, HKV, seed=2, local_blocks=2)
+    q1, k1, v1 = (x.clone().requires_grad_() for x in (q, k, v))
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, k, v))
+    o = topk_sparse_attention(q1, k1, v1, idx, BS, cu)
+    want = oracle.topk_sparse_attention(qf, kf, vf, idx, BS, cu)
+    assert_close(o, want, "o")
+    o.backward(do)
+    want.backward(do.float())
+    _grads_close((("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)))
+    wp = torch.softmax(torch.randn(HKV, KS, generator=g, device=device), -1).bfloat16()
+    ck, ccu = weightedpool_compress(k, wp, cu, KS, ST)
+    cv, _ = weightedpool_compress(v, wp, cu, KS, ST)
+    max_c = int((ccu[1:] - ccu[:-1]).max())
+    q1, k1, v1 = (x.clone().requires_grad_() for x in (q, ck, cv))
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, ck, cv))
+    o, sel = compressed_attention(q1, k1, v1, KS, ST, BS, TOPK, cu, ccu, max(lens), max_c, None, 1, 2)
+    want, want_sel = oracle.compressed_attention(qf, kf, vf, KS, ST, BS, TOPK, cu, ccu, max(lens), max_c, None, 1, 2)
+    assert_close(o, want, "o")
+    assert torch.equal(sel, want_sel)
+    o.backward(do)
+    want.backward(do.float())
+    _grads_close((("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)))
