@@ -96,9 +96,11 @@ class NativeSparseAttention(torch.nn.Module):
         compressed_k = self.rope(compressed_k, compressed_cu_seqlens, stride=self.kernel_stride)
 
         compressed_seqlens = compressed_cu_seqlens[1:] - compressed_cu_seqlens[:-1]
+        # the two maxima the reference reads back one by one (:197-198), in one device read
+        max_seqlen, max_compressed = torch.stack((seqlens.max(), compressed_seqlens.max())).tolist()
         compressed_attn_output, topk_idx = compressed_attention(
             q, compressed_k, compressed_v, self.kernel_size, self.kernel_stride, self.block_size, self.topk, cu_seqlens,
-            compressed_cu_seqlens, seqlens.max().item(), compressed_seqlens.max().item(), None, self.init_blocks, self.local_blocks)
+            compressed_cu_seqlens, max_seqlen, max_compressed, None, self.init_blocks, self.local_blocks)
 
         k = self.rope(k, cu_seqlens)
         sparse_attn_output = topk_sparse_attention(q, k, v, topk_idx, self.block_size, cu_seqlens, None)
