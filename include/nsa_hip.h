@@ -66,7 +66,9 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
  *   receive the "KV block -> queries" reverse index built on the way:
  *     segments = nsa_topk_reverse_index_segments(); segment s = kv_head*(T/block+batch) + global block;
  *     out_segment_offsets int32 [segments+1]; out_queries int32 [Hkv*T*topk], the tokens of
- *     segment s are out_queries[off[s] : off[s+1]], ascending.
+ *     segment s are out_queries[off[s] : off[s+1]], ascending.  For block_size 256 the index (and the
+ *     dK/dV pass) works on the four 64-key pieces of every block: read `block` as 64 above, out_queries
+ *     then holds up to 4*Hkv*T*topk entries, and a query appears under the pieces at or before its position.
  * dK/dV are reduced in a fixed order (no atomics): results are run-to-run deterministic.
  * phases: NSA_BWD_PHASE_ALL, or a subset to re-run single passes on a workspace that an
  * earlier call with identical arguments has already filled (PREP = delta + reverse index).

@@ -28,14 +28,20 @@ struct BwdLayout {
   int64_t max_blocks, n_pairs, max_items, n_slots;
 };
 
-static constexpr int LIST_CHUNK = 768;  // queries per dK/dV work item in big launches
+static constexpr int LIST_CHUNK = 768;
+
+// Key block of the dK/dV pass.  Blocks of 256 keys are handled as four 64-key blocks (one reverse-index entry per
+// query and 64-key piece at or before the query's position): the 256-key variant of the kernel needs more registers
+// than a wave has (it spilled inside its loop and took 9 ms where the 64-key variant takes 3).
+constexpr int dkdv_block(int bs) { return bs >= 256 ? 64 : bs; }  // queries per dK/dV work item in big launches
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t topk, int64_t bs) {
   BwdLayout L;
-  L.max_blocks = T / bs + B;  // every sequence adds at most one ragged block
-  L.n_pairs = Hkv * T * topk;
+  const int64_t ebs = dkdv_block((int)bs);
+  L.max_blocks = T / ebs + B;  // every sequence adds at most one ragged block
+  L.n_pairs = Hkv * T * topk * (bs / ebs);
   const int chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
   L.max_items = (L.n_pairs + chunk - 1) / chunk + Hkv * L.max_blocks;
   size_t tmp = 0;
@@ -57,7 +63,7 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.n_slots = nsa_chunk_slots(T, B);
   L.kf = take(retile_bytes(T, B, Hkv, D));   // row-fragment copies of K and V for the dQ pass
   L.vf = take(retile_bytes(T, B, Hkv, D));
-  L.partial = take((size_t)L.max_items * bs * D * 4 * 2);
+  L.partial = take((size_t)L.max_items * ebs * D * 4 * 2);
   L.total = off;
   return L;
 }
@@ -70,19 +76,23 @@ __global__ __launch_bounds__(256) void seq_blocks_kernel(const int32_t* __restri
 
 __global__ __launch_bounds__(256) void emit_pairs_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ cu,
                                                          const int32_t* __restrict__ cu_blk, int batch, int total_len, int Hkv,
-                                                         int topk, int bs, int max_blocks, long long ish, long long isn,
+                                                         int topk, int bs, int ebs, int max_blocks, long long ish, long long isn,
                                                          long long isk, uint32_t* __restrict__ keys, int32_t* __restrict__ vals) {
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // (h, t, e), e fastest
-  const long long n = (long long)Hkv * total_len * topk;
+  // one thread per (head, token, entry, piece of ebs keys inside the selected block); bs == ebs: one piece
+  const int sub = bs / ebs;
+  const long long n = (long long)Hkv * total_len * topk * sub;
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
-  const int e = (int)(i % topk);
-  const int t = (int)((i / topk) % total_len);
-  const int h = (int)(i / ((long long)topk * total_len));
+  const int s = (int)(i % sub);
+  const int e = (int)((i / sub) % topk);
+  const int t = (int)((i / ((long long)sub * topk)) % total_len);
+  const int h = (int)(i / ((long long)sub * topk * total_len));
   const int b = find_sequence(cu, batch, t);
-  const int qb = (t - cu[b]) / bs;
+  const int pos = t - cu[b];
   const int blk = idx[(long long)h * ish + (long long)t * isn + (long long)e * isk];
-  const bool ok = blk >= 0 && blk <= qb;
-  keys[i] = ok ? (uint32_t)(h * max_blocks + cu_blk[b] + blk) : (uint32_t)(Hkv * max_blocks);
+  const int piece = blk * sub + s;
+  const bool ok = blk >= 0 && blk <= pos / bs && piece * ebs <= pos;  // pieces wholly after the query hold nothing it sees
+  keys[i] = ok ? (uint32_t)(h * max_blocks + cu_blk[b] + piece) : (uint32_t)(Hkv * max_blocks);
   vals[i] = t;
 }
 
@@ -275,9 +285,10 @@ static int build_reverse_index(const BwdArgs& a, const BwdLayout& L) {
   int32_t* seg_off = (int32_t*)(ws + L.seg_off);
   int32_t* chunk_off = (int32_t*)(ws + L.chunk_off);
   const int n_seg = (int)(a.Hkv * L.max_blocks);
-  seq_blocks_kernel<<<1, 256, 0, a.stream>>>(a.cu, (int)a.B, (int)a.bs, cu_blk);
+  seq_blocks_kernel<<<1, 256, 0, a.stream>>>(a.cu, (int)a.B, dkdv_block((int)a.bs), cu_blk);
   emit_pairs_kernel<<<(unsigned)((L.n_pairs + 255) / 256), 256, 0, a.stream>>>(
-      a.idx, a.cu, cu_blk, (int)a.B, (int)a.T, (int)a.Hkv, (int)a.topk, (int)a.bs, (int)L.max_blocks, a.ish, a.isn, a.isk, keys_in, vals_in);
+      a.idx, a.cu, cu_blk, (int)a.B, (int)a.T, (int)a.Hkv, (int)a.topk, (int)a.bs, dkdv_block((int)a.bs), (int)L.max_blocks, a.ish, a.isn, a.isk,
+      keys_in, vals_in);
   unsigned bits = 1;
   while ((1ull << bits) <= (unsigned long long)n_seg) bits++;
   size_t tmp = L.sort_tmp_bytes;
@@ -334,10 +345,10 @@ static int run_bwd(const BwdArgs& a) {
     p.qsn = (int)a.qsn; p.qsh = (int)a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = (int)a.dsn; p.dsh = (int)a.dsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1; p.window = -1;
     p.chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
-    constexpr int NT = 64 * dkdv_waves(BS);
-    if (GT == 1) dkdv_kernel<T, D, BS, false, true><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
-    else dkdv_kernel<T, D, BS, false, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
-    dkdv_reduce_kernel<T, D, BS><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(
+    constexpr int EBS = dkdv_block(BS), NT = 64 * dkdv_waves(EBS);
+    if (GT == 1) dkdv_kernel<T, D, EBS, false, true><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
+    else dkdv_kernel<T, D, EBS, false, false><<<(unsigned)L.max_items, NT, 0, a.stream>>>(p);
+    dkdv_reduce_kernel<T, D, EBS><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(
         p.partial, p.chunk_off, a.cu, p.cu_blk, (int)a.B, (int)L.max_blocks, (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
   }
   return nsa_check_launch();
@@ -370,7 +381,7 @@ extern "C" size_t nsa_topk_attn_bwd_workspace_bytes(int64_t total_len, int64_t b
 }
 
 extern "C" int64_t nsa_topk_reverse_index_segments(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t block_size) {
-  return num_kv_heads * (total_len / block_size + batch);
+  return num_kv_heads * (total_len / dkdv_block((int)block_size) + batch);
 }
 
 extern "C" int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,

@@ -77,7 +77,8 @@ def _topk_sparse_attention_bwd(o, do, lse, q, k, v, topk_idx, block_size, cu_seq
     if return_reverse_index:
         n_seg = lib.nsa_topk_reverse_index_segments(q_len, batch, num_k_heads, block_size)
         seg_off = torch.empty(n_seg + 1, dtype=torch.int32, device=q.device)
-        queries = torch.empty(num_k_heads * q_len * topk, dtype=torch.int32, device=q.device)
+        pieces = 4 if block_size == 256 else 1  # the index of 256-key blocks is kept per 64-key piece
+        queries = torch.empty(pieces * num_k_heads * q_len * topk, dtype=torch.int32, device=q.device)
     rc = lib.nsa_topk_attn_bwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(), topk_idx.data_ptr(),
         cu_seqlens_q.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), q_len, batch, num_q_heads, num_k_heads,
