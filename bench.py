@@ -315,6 +315,8 @@ def main():
         print("bench.py measures one GPU: the operator path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
 
+    import __graft_entry__
+    __graft_entry__.ensure_built()  # uses the library that is built; compiles only in a tree without one
     from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
     from native_sparse_attention.testing import cu_from_lens, make_topk_idx
     from native_sparse_attention import _lib
