@@ -316,7 +316,7 @@ def main():
         sys.exit(2)
 
     import __graft_entry__
-    __graft_entry__.ensure_built()  # uses the library that is built; compiles only in a tree without one
+    __graft_entry__.ensure_built()  # uses the library that is built; compiles only when it is missing or older than its sources
     from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
     from native_sparse_attention.testing import cu_from_lens, make_topk_idx
     from native_sparse_attention import _lib

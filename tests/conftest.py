@@ -12,7 +12,7 @@ for p in (ROOT, PKG):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
-    # the tests load the library that is built; only a tree without one is built first
+    # the tests load the library that is built; a missing or out-of-date one is (re)built first
     import __graft_entry__
     __graft_entry__.ensure_built()
 
