@@ -12,7 +12,7 @@
  *  - Varlen tensors are [total_len, heads, head_dim]; cu_seqlens is int32 [batch+1].
  *  - sm_scale of the prefill/training attention entry points must be positive (NSA_ERR_UNSUPPORTED otherwise).
  *  - Return value: NSA_OK (0) or a negative NSA_ERR_* code; nothing is launched on error.
- *  - Re-entrant: no global state.
+ *  - Re-entrant: no global state (one exception, stated there: nsa_topk_decode_static).
  */
 #ifndef NSA_HIP_H
 #define NSA_HIP_H
@@ -332,6 +332,20 @@ int nsa_topk_decode(const void* q, const void* k, const void* v, const int32_t* 
                     int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len, int64_t topk,
                     int64_t block_size, const int64_t* strides, float sm_scale, int dtype, void* workspace,
                     size_t workspace_bytes, void* stream);
+/* nsa_topk_decode_static: nsa_topk_decode for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * arguments and results as nsa_topk_decode, without the workspace: the split-K partials live in a device array
+ * of NSA_TOPK_DECODE_STATIC_MAX_BYTES that the library holds on every GPU it runs on until the process ends
+ * (this entry point is the library's one piece of global state).  Returns NSA_ERR_WORKSPACE, and launches
+ * nothing, when nsa_topk_decode_workspace_bytes(...) of the call exceeds that size.  All calls on one GPU share
+ * the array: calls that may overlap on one GPU (different streams, different threads) race and must be
+ * serialised by the caller.  Nothing is allocated, freed or cleared; the first call on a device looks the
+ * array's address up (make that call outside a graph capture).
+ */
+#define NSA_TOPK_DECODE_STATIC_MAX_BYTES (4u << 20)
+int nsa_topk_decode_static(const void* q, const void* k, const void* v, const int32_t* topk_idx, const int32_t* seqlens, void* o,
+                           int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t slab_len,
+                           int64_t topk, int64_t block_size, const int64_t* strides, float sm_scale, int dtype, void* stream);
 /* nsa_cmp_decode replaces the torch-op chain of compressed_attention_decode
  * (native_sparse_attention/ops/torch/compressed_attention_decode.py:65-153, with transform_score :21-62):
  * attention over the first compress_seqlens[b] rows of the compressed slab, then (if out_topk_idx is

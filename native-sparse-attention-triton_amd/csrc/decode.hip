@@ -10,6 +10,7 @@
 // selected-block and the sliding-window branch share one partial launch, and one launch does both merges and
 // the gated sum with the compressed branch; the compressed branch's merge runs inside its block-selection kernel.
 #include "nsa_common.h"
+#include <mutex>
 #include <type_traits>
 
 struct DecodeParams {
@@ -522,6 +523,48 @@ extern "C" int nsa_topk_decode(const void* q, const void* k, const void* v, cons
 #define CALL(T, D) run_decode<T, D>(1, p, o, osb, osh, nullptr, (char*)workspace, s)
   DECODE_DISPATCH(CALL)
 #undef CALL
+}
+
+// ------------------------------------------------------------------------------------------
+// nsa_topk_decode for callers that cannot allocate: the split-K partials live in a file-scope device array
+// instead of a caller workspace.  Every GPU the library runs on holds its own copy of the array until the
+// process ends; its device address is looked up once per device (the array's name in host code is only a
+// handle for that lookup, never an address a kernel may be given).
+static constexpr size_t STATIC_SCRATCH_BYTES = NSA_TOPK_DECODE_STATIC_MAX_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+static constexpr int STATIC_MAX_DEVICES = 64;
+static void* scratch_addr[STATIC_MAX_DEVICES];   // per device, filled on the first call with that device current
+static std::mutex scratch_mutex;
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return NSA_ERR_LAUNCH;
+  std::lock_guard<std::mutex> hold(scratch_mutex);
+  if (!scratch_addr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return NSA_ERR_LAUNCH;
+    scratch_addr[dev] = ptr;
+  }
+  *out = scratch_addr[dev];
+  return NSA_OK;
+}
+
+extern "C" int nsa_topk_decode_static(const void* q, const void* k, const void* v, const int32_t* topk_idx, const int32_t* seqlens,
+                                      void* o, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                      int64_t slab_len, int64_t topk, int64_t block_size, const int64_t* strides, float sm_scale,
+                                      int dtype, void* stream) {
+  if (batch <= 0 || num_kv_heads <= 0 || num_q_heads <= 0 || num_q_heads % num_kv_heads != 0 || topk <= 0) return NSA_ERR_BAD_ARG;
+  if (block_size != 32 && block_size != 64 && block_size != 128 && block_size != 256) return NSA_ERR_UNSUPPORTED;
+  // sizes whose partials do not fit the array are refused before anything is looked up or launched
+  if (nsa_topk_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, topk, block_size) > STATIC_SCRATCH_BYTES)
+    return NSA_ERR_WORKSPACE;
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != NSA_OK) return rc;
+  // the partial kernel writes every (m, l, O) slot the merge kernel reads, so nothing left behind by an
+  // earlier call needs clearing
+  return nsa_topk_decode(q, k, v, topk_idx, seqlens, o, batch, num_q_heads, num_kv_heads, head_dim, slab_len, topk, block_size,
+                         strides, sm_scale, dtype, ws, STATIC_SCRATCH_BYTES, stream);
 }
 
 static size_t cmp_decode_partial(int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t slab_len) {

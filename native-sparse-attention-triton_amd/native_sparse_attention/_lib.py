@@ -30,6 +30,7 @@ _SIGNATURES = {
     "nsa_dense_decode": (c_int, [P] * 5 + [I] * 5 + [P, F, c_int, P, Z, P]),
     "nsa_topk_decode_workspace_bytes": (Z, [I] * 6),
     "nsa_topk_decode": (c_int, [P] * 6 + [I] * 7 + [P, F, c_int, P, Z, P]),
+    "nsa_topk_decode_static": (c_int, [P] * 6 + [I] * 7 + [P, F, c_int, P]),
     "nsa_cmp_decode_workspace_bytes": (Z, [I] * 5),
     "nsa_cmp_decode": (c_int, [P] * 7 + [I] * 12 + [P, F, c_int, P, Z, P]),
     "nsa_cmp_attn_fwd": (c_int, [P] * 7 + [I] * 8 + [P, F, c_int, P]),
