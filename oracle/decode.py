@@ -54,19 +54,21 @@ def topk_sparse_attention_decode(q, k, v, topk_idx, block_size, seqlens, sm_scal
 
 def compressed_attention_decode(
     q, k, v, seqlens, compress_seqlens, kernel_size, kernel_stride, block_size, topk,
-    init_blocks: int = 1, local_blocks: int = 2, sm_scale: Optional[float] = None,
+    init_blocks: int = 1, local_blocks: int = 2, sm_scale: Optional[float] = None, return_scores: bool = False,
 ):
     """compressed_attention_decode.py:65-153.
 
     Returns (out [B,Hq,d], topk_idx [Hkv,B,min(topk, ceil(max(seqlens)/block))] int32);
-    an empty compressed slab gives zeros and a [Hkv,B,1] zero index (:105-108).
+    an empty compressed slab gives zeros and a [Hkv,B,1] zero index (:105-108).  With ``return_scores`` the
+    block scores [Hkv,B,max_blocks] the ids were taken from are returned as well (None for an empty slab).
     """
     assert block_size % kernel_size == 0 and kernel_size % kernel_stride == 0
     B, Hq, d = q.shape
     L, Hkv = k.shape[1], k.shape[2]
     scale = 1.0 / math.sqrt(d) if sm_scale is None else sm_scale
     if L == 0:
-        return torch.zeros_like(q), torch.zeros(Hkv, B, 1, dtype=torch.int32, device=q.device)
+        empty = (torch.zeros_like(q), torch.zeros(Hkv, B, 1, dtype=torch.int32, device=q.device))
+        return empty + (None,) if return_scores else empty
     vis = torch.arange(L, device=q.device)[None, :] < compress_seqlens[:, None].to(torch.int64)
     o, p = _attend(q, k, v, vis[:, None, :].expand(B, Hkv, L), scale)
     score = p.float().sum(2).permute(1, 0, 2)                        # [Hkv, B, L]
@@ -87,4 +89,4 @@ def compressed_attention_decode(
     kk = min(topk, max_blocks)
     idx = bscore.topk(kk, dim=-1).indices.sort(-1).values
     idx = torch.where(idx > qb[None, :, None], torch.full_like(idx, -1), idx)
-    return o, idx.to(torch.int32)
+    return (o, idx.to(torch.int32), bscore) if return_scores else (o, idx.to(torch.int32))

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import assert_close
+from helpers import assert_close, assert_ids_match
 from native_sparse_attention.ops import compressed_attention_decode, flash_attention_decode, topk_sparse_attention_decode
 from native_sparse_attention.testing import cu_from_lens, make_topk_idx
 
@@ -82,12 +82,11 @@ def test_compressed_decode(device, lens, Hq, Hkv, d, topk, dtype):
     slab = max(int(clens.max()), 1) + 3
     q, k, v = _slabs(B, slab, Hq, Hkv, d, dtype, device)
     o, idx = compressed_attention_decode(q, k, v, seqlens, clens, ks, st, bs, topk)
-    want_o, want_idx = oracle.compressed_attention_decode(q.float(), k.float(), v.float(), seqlens, clens, ks, st, bs, topk)
+    want_o, want_idx, bscore = oracle.compressed_attention_decode(q.float(), k.float(), v.float(), seqlens, clens, ks, st, bs, topk,
+                                                                  return_scores=True)
     assert_close(o, want_o, "o")
-    assert idx.dtype == torch.int32 and idx.shape == want_idx.shape
-    # structural invariants + exact match wherever the oracle's k-th and (k+1)-th block scores differ
-    mism = (idx != want_idx).any(-1)
-    assert mism.float().mean().item() <= 0.05, "topk ids differ on %.1f%% of rows" % (100 * mism.float().mean().item())
+    # exact match wherever the oracle's k-th and (k+1)-th block scores differ by more than 1e-3, then structural invariants
+    assert_ids_match(idx, want_idx, bscore, (seqlens.long() - 1) // bs, "decode topk_idx", min_overlap=0.9)
     for b, L in enumerate(lens):
         qb = (L - 1) // bs
         for h in range(Hkv):

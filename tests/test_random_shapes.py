@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import assert_close
+from helpers import assert_close, assert_ids_match
 from native_sparse_attention.ops import compressed_attention, flash_attention_varlen, topk_sparse_attention, weightedpool_compress
 from native_sparse_attention.ops.sliding_window import sliding_window_attention_varlen
 from native_sparse_attention.testing import cu_from_lens, make_topk_idx
@@ -76,9 +76,10 @@ def test_random_shapes(device, seed):
             q1, k1, v1 = q.clone().requires_grad_(), ck.detach().clone().requires_grad_(), cv.detach().clone().requires_grad_()
             o, idx = compressed_attention(q1, k1, v1, ks, st, bs, topk, cu, ccu, max(lens), max_c, None, 1, 2)
             qf, kf, vf = q.float().requires_grad_(), ck.detach().float().requires_grad_(), cv.detach().float().requires_grad_()
-            want, want_idx = oracle.compressed_attention(qf, kf, vf, ks, st, bs, topk, cu, ccu, max(lens), max_c, None, 1, 2)
-            # rows may differ where two block scores tie within rounding; the tests with a decision margin are elsewhere
-            assert (idx != want_idx).any(-1).float().mean().item() <= 0.02
+            want, want_idx, bscore = oracle.compressed_attention(qf, kf, vf, ks, st, bs, topk, cu, ccu, max(lens), max_c, None, 1, 2,
+                                                                 return_scores=True)
+            qb = torch.cat([torch.arange(L, device=device) for L in lens]) // bs
+            assert_ids_match(idx, want_idx, bscore, qb, "topk_idx", min_overlap=0.9)
         o.backward(do)
         want.backward(do.float())
         assert_close(o, want, "o")
@@ -121,9 +122,10 @@ def test_random_decode_shapes(device, seed):
         ck, cv = cache[0, :B, :cslab], cache[1, :B, :cslab]
         k_sel = rng.randint(1, 8)
         o_cmp, sel = compressed_attention_decode(q, ck, cv, seqlens, clens, ks, st, cbs, k_sel)
-        want_cmp, want_sel = oracle.compressed_attention_decode(q.float(), ck.float(), cv.float(), seqlens, clens, ks, st, cbs, k_sel)
+        want_cmp, want_sel, bscore = oracle.compressed_attention_decode(q.float(), ck.float(), cv.float(), seqlens, clens, ks, st, cbs,
+                                                                        k_sel, return_scores=True)
         assert_close(o_cmp, want_cmp, "cmp o")
-        assert sel.shape == want_sel.shape and (sel != want_sel).any(-1).float().mean().item() <= 0.1
+        assert_ids_match(sel, want_sel, bscore, (seqlens.long() - 1) // cbs, "decode ids", min_overlap=0.8)
         W = min(slab, rng.choice([16, 64, 512]))
         wk, wv = cache[0, 1:B + 1, :W], cache[1, 1:B + 1, :W]
         wlen = torch.tensor([min(L, W) for L in lens], dtype=torch.int32, device=device)
