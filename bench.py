@@ -27,7 +27,7 @@ HQ, HKV, D, BS = 64, 4, 128, 64
 H100_FWD_BWD_MS = 12.417 + 15.154
 # memory-side traffic per launch at the default workload (N=32768, top16), bytes: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, scaled by what the same counters read for a plain 1 GiB copy (x2.0 and x1.0); see profiles/
-MEASURED_TRAFFIC = {"fwd_attend": 15.8 * 2**30, "bwd_dq": 17.0 * 2**30, "bwd_dkdv": 18.3 * 2**30}
+MEASURED_TRAFFIC = {"topk_fwd_kernel": 15.8 * 2**30, "dq_kernel": 17.0 * 2**30, "dkdv_kernel": 18.3 * 2**30}
 
 
 def _events_ms(fn, iters):
@@ -42,32 +42,34 @@ def _events_ms(fn, iters):
 
 
 def cpu_baseline():
-    """Oracle (pure PyTorch restatement) on the host cores, on a bounded sample of the headline workload: the same
-    heads and selection (64 q / 4 kv heads, d=128, block 64, top-16, fp32) on one 4096-token sequence, forward +
-    backward; two runs of several seconds each, the faster one reported."""
+    """The oracle (this repository's restatement of the reference's ops/torch/topk_sparse_attention.py:19-83) on the
+    host cores, on the reference's CPU-runnable configuration: fp32, cu_seqlens = [0, 512, 1536, 2048], 16 query heads,
+    1 KV head, head_dim 64, block 64, top-8 with block 0 and the query's own block forced, q / k / v drawn in that order
+    from torch.manual_seed(0); forward only, one warm-up, median of 7 runs, every host core torch was given.  `value`
+    is in the unit of the headline metric (TFLOP/s on selected-block FLOPs)."""
     sys.path.insert(0, ROOT)
+    import statistics
+
     import oracle
     from native_sparse_attention.testing import cu_from_lens, make_topk_idx
 
     torch.manual_seed(0)
-    n = 4096
-    cu = cu_from_lens([n])
-    q, k, v = (torch.randn(n, h, 128, requires_grad=True) for h in (64, 4, 4))
-    idx = make_topk_idx(cu, 64, 16, 4, seed=0, local_blocks=2)
-    do = torch.randn(n, 64, 128)
-    flops = 3.5 * 4 * 128 * 64 * 16 * int((idx >= 0).sum())
+    cu = cu_from_lens([512, 1024, 512])
+    q, k, v = torch.randn(2048, 16, 64), torch.randn(2048, 1, 64), torch.randn(2048, 1, 64)
+    idx = make_topk_idx(cu, 64, 8, 1, seed=0, local_blocks=1)
+    flops = 4.0 * 64 * 64 * 16 * int((idx >= 0).sum())
     times = []
-    for _ in range(2):
-        t0 = time.perf_counter()
-        oracle.topk_sparse_attention(q, k, v, idx, 64, cu).backward(do)
-        times.append(time.perf_counter() - t0)
-        q.grad = k.grad = v.grad = None
-    best = min(times)
+    with torch.no_grad():
+        for i in range(8):
+            t0 = time.perf_counter()
+            oracle.topk_sparse_attention(q, k, v, idx, 64, cu)
+            if i > 0:
+                times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
     return {
-        "value": flops / best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "ms": best * 1e3,
-        "sample": "oracle forward+backward fp32 on one 4096-token sequence of the headline shape (64q/4kv heads, d=128, block 64, "
-                  "top-16); best of 2 runs",
+        "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port", "ms": med * 1e3,
+        "sample": "oracle forward, fp32, cu_seqlens=[0,512,1536,2048], 16 q / 1 kv heads, d=64, block 64, top-8 "
+                  "(block 0 and own block forced), seed 0; 1 warm-up, median of 7 runs",
     }
 
 
@@ -296,6 +298,62 @@ def bench_layer(args, dev):
     }
 
 
+def measure_topk(N, topk, steps, warmup, dev, per_kernel):
+    """One point of the top-k sweep: forward + backward of topk_sparse_attention on a single sequence of N tokens (64 q / 4 kv
+    heads, d=128, block 64), inputs resident in HBM.  ms_per_step: wall clock over `steps` steps after `warmup`; fwd_ms /
+    bwd_ms and (per_kernel) the duration of every kernel of the step: HIP events on the launch stream, single passes
+    re-run on filled workspaces."""
+    from native_sparse_attention import _lib
+    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
+    from native_sparse_attention.testing import cu_from_lens, make_topk_idx
+
+    G = HQ // HKV
+    g = torch.Generator(device=dev).manual_seed(0)
+    cu = cu_from_lens([N], dev)
+    q = torch.randn(N, HQ, D, generator=g, device=dev).bfloat16()
+    k = torch.randn(N, HKV, D, generator=g, device=dev).bfloat16()
+    v = torch.randn(N, HKV, D, generator=g, device=dev).bfloat16()
+    do = torch.randn(N, HQ, D, generator=g, device=dev).bfloat16()
+    idx = make_topk_idx(cu, BS, topk, HKV, seed=0, local_blocks=2)
+    sm = D ** -0.5
+    n_pairs = int((idx >= 0).sum())
+    f_fwd = 4.0 * D * BS * G * n_pairs
+
+    def step():
+        o, lse = _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm)
+        return _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    lib = _lib.load()
+    ws_f = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, HKV, D), dev)
+    ws_b = _lib.workspace(lib.nsa_topk_attn_bwd_workspace_bytes(N, 1, HQ, HKV, D, topk, BS), dev)
+    o, lse = _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_f)
+    grads = _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_b)
+    it = max(3, min(steps, 20))
+    fwd = lambda ph: _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_f, phases=ph, out=(o, lse))
+    bwd = lambda ph: _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_b, phases=ph, out=grads)
+    out = {"f_fwd": f_fwd, "ms_per_step": ms_per_step, "fwd_ms": _events_ms(lambda: fwd(3), it), "bwd_ms": _events_ms(lambda: bwd(7), it)}
+    if per_kernel:
+        qb, kvb = q.numel() * 2, k.numel() * 2                 # bytes of one [N,64,128] and of one [N,4,128] tensor
+        small = idx.numel() * 4 + 2 * HQ * N * 4               # block ids, lse / delta
+        out["kernels"] = {
+            # name: (ms, algorithmic FLOPs per launch, bytes the kernel must read or write at least once)
+            "topk_fwd_kernel": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd, 2 * qb + 2 * kvb + small),              # QK^T, PV
+            "dq_kernel": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd, 4 * qb + 2 * kvb + small),                   # dS K (recomputed QK^T, dO V^T not counted)
+            "dkdv_kernel": (_events_ms(lambda: bwd(2), it), 2.0 * f_fwd, 2 * qb + 4 * kvb + small),       # QK^T, dO V^T, P^T dO, dS^T Q
+            "reverse_index": (_events_ms(lambda: bwd(1), it) , 0.0, None),   # run alone this phase also holds the stand-alone delta pass
+        }
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -304,6 +362,7 @@ def main():
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--topk", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the N x top-k sweep table (config.sweep)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 1 GiB device copies (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--readme-heads", action="store_true",
@@ -317,10 +376,6 @@ def main():
 
     import __graft_entry__
     __graft_entry__.ensure_built()  # uses the library that is built; compiles only when it is missing or older than its sources
-    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
-    from native_sparse_attention.testing import cu_from_lens, make_topk_idx
-    from native_sparse_attention import _lib
-
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload != "topk":
@@ -328,76 +383,51 @@ def main():
         print(json.dumps(fn(args, dev)))
         return
     N, topk = args.seqlen, args.topk
-    G = HQ // HKV
-    g = torch.Generator(device=dev).manual_seed(0)
-    cu = cu_from_lens([N], dev)
-    q = torch.randn(N, HQ, D, generator=g, device=dev).bfloat16()
-    k = torch.randn(N, HKV, D, generator=g, device=dev).bfloat16()
-    v = torch.randn(N, HKV, D, generator=g, device=dev).bfloat16()
-    do = torch.randn(N, HQ, D, generator=g, device=dev).bfloat16()
-    idx = make_topk_idx(cu, BS, topk, HKV, seed=0, local_blocks=2)
-    sm = D ** -0.5
-    f_fwd = 4.0 * D * BS * G * int((idx >= 0).sum())
+    r = measure_topk(N, topk, args.steps, args.warmup, dev, per_kernel=True)
+    f_fwd, ms_per_step, kern = r["f_fwd"], r["ms_per_step"], r["kernels"]
     f_total = 3.5 * f_fwd
-
-    def step():
-        o, lse = _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm)
-        return _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    # per-kernel durations, HIP events on the launch stream; single passes re-run on filled workspaces
-    lib = _lib.load()
-    ws_f = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, HKV, D), dev)
-    ws_b = _lib.workspace(lib.nsa_topk_attn_bwd_workspace_bytes(N, 1, HQ, HKV, D, topk, BS), dev)
-    o, lse = _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_f)
-    grads = _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_b)
-    it = max(3, min(args.steps, 20))
-    fwd = lambda ph: _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_f, phases=ph, out=(o, lse))
-    bwd = lambda ph: _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_b, phases=ph, out=grads)
-    kern = {
-        "fwd_attend": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd),        # QK^T, PV
-        # preparation run alone: delta pass + reverse index.  In a full backward the delta pass does not run (dQ
-        # forms delta from the dO rows it holds), so kernel_ms adds up to more than bwd_ms
-        "bwd_prep": (_events_ms(lambda: bwd(1), it), 0.0),
-        "bwd_index_and_dq": (_events_ms(lambda: bwd(5), it), 0.0),         # reverse index + dQ with delta formed inside
-        "bwd_dkdv": (_events_ms(lambda: bwd(2), it), 2.0 * f_fwd),          # QK^T, dO V^T, P^T dO, dS^T Q
-        "bwd_dq": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd),            # dS K (its recomputed QK^T, dO V^T are not counted)
-    }
-    fwd_ms = _events_ms(lambda: fwd(3), it)
-    bwd_ms = _events_ms(lambda: bwd(7), it)
-    # the three MFMA kernels take about a third of the step each (which one is slowest changes from run to run);
-    # the roofline object describes the one that owns most of the algorithmic FLOPs (4 of the 7 matmuls)
-    dom = max(kern, key=lambda n: kern[n][1])
-    dom_ms, dom_flops = kern[dom]
-    achieved = dom_flops / dom_ms / 1e9
+    headline = (N, topk) == (32768, 16)
+    kernels = []
+    for name, (ms, flops, unique) in kern.items():
+        traffic = MEASURED_TRAFFIC.get(name) if headline else None
+        kernels.append({
+            "kernel": name, "ms": ms, "algorithmic_flops": flops, "tflops": flops / ms / 1e9 if flops else None,
+            "frac": flops / ms / 1e9 / PEAK_BF16_TFLOPS if flops else None,
+            "unique_bytes": unique, "traffic": traffic, "traffic_over_unique": traffic / unique if traffic and unique else None,
+        })
+    mfma = [x for x in kernels if x["algorithmic_flops"]]
+    dom = max(mfma, key=lambda x: x["ms"])   # the kernel that takes the most time
     line = {
         "metric": "topk_sparse_attn fwd+bwd TFLOP/s on selected-block FLOPs (N=%d, top%d)" % (N, topk),
         "value": f_total / ms_per_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": (H100_FWD_BWD_MS / ms_per_step) if (N, topk) == (32768, 16) else None,
+        "vs_baseline": (H100_FWD_BWD_MS / ms_per_step) if headline else None,
         "dtype": "bf16", "data": "synthetic",
         "config": {
             "workload": "topk_sparse_attention fwd+bwd, single sequence N=%d, 64 q / 4 kv heads, d=128, block 64, top-%d, "
                         "causal topk_idx with block 0 and two local blocks forced" % (N, topk),
             "baseline": "H100 Triton fwd+bwd ms published in the reference README (12.417 + 15.154)",
-            "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "frac_of_bf16_peak": f_total / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
-            "kernel_ms": {n: kern[n][0] for n in kern},
-            "kernel_tflops": {n: kern[n][1] / kern[n][0] / 1e9 for n in kern if kern[n][1] > 0},
+            "fwd_ms": r["fwd_ms"], "bwd_ms": r["bwd_ms"], "frac_of_bf16_peak": f_total / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
         },
         "roofline": {
-            "bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / PEAK_BF16_TFLOPS,
-            "traffic": MEASURED_TRAFFIC.get(dom) if (N, topk) == (32768, 16) else None,
+            "bound": "mfma", "kernel": dom["kernel"], "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+            "frac": dom["frac"], "traffic": dom["traffic"], "unique_bytes": dom["unique_bytes"],
+            "traffic_over_unique": dom["traffic_over_unique"],
+            "note": "kernel = the MFMA kernel with the largest measured duration; achieved = its algorithmic FLOPs per launch / "
+                    "its duration (HIP events on the launch stream); traffic = L2<->memory-side bytes per launch from rocprofv3 "
+                    "--pmc FETCH_SIZE / WRITE_SIZE (profiles/), unique_bytes = what the kernel must read and write at least once",
+            "step_frac": f_total / ms_per_step / 1e9 / PEAK_BF16_TFLOPS,
+            "kernels": kernels,
         },
     }
+    if not args.no_sweep:
+        sweep = []
+        for n in (2048, 4096, 8192, 16384, 32768, 65536):
+            for kk in (8, 16):
+                m = r if (n, kk) == (N, topk) else measure_topk(n, kk, max(3, min(args.steps, 10)), 2, dev, per_kernel=False)
+                sweep.append({"N": n, "topk": kk, "fwd_ms": round(m["fwd_ms"], 4), "bwd_ms": round(m["bwd_ms"], 4),
+                              "fwd_bwd_ms": round(m["ms_per_step"], 4), "tflops": round(3.5 * m["f_fwd"] / m["ms_per_step"] / 1e9, 1)})
+        line["config"]["sweep"] = sweep
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)

@@ -569,7 +569,11 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
           xprev = xs;
           const int blk = c / rr;
           if ((li & (min(rr, 16) - 1)) == 0 && blk < p.full_blocks && blk < p.nb_row)
-            atomicAdd(&bs_s[(4 * wave + lg) * p.nb_row + blk], z);  // LDS add without return: nothing waits for it
+            // LDS add without return: nothing waits for it.  Row 4 * wave + lg belongs to this wave alone and an
+            // instruction holds at most one lane per (row, block), so all additions to one address come from one
+            // wave in program order (head tiles, then chunks): the sum, and with it the selection, is the same
+            // on every run
+            atomicAdd(&bs_s[(4 * wave + lg) * p.nb_row + blk], z);
         }
       }
       if (ch + 1 < n_chunks) stg.stash(k_s[buf ^ 1], k_s[buf ^ 1], tid);

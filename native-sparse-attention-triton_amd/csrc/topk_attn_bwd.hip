@@ -2,9 +2,11 @@
 //
 // Passes, all on the caller's stream and out of the caller's workspace (run in the order 1, 3, 2: the dQ
 // pass leaves delta behind for the dK/dV pass):
-//   1. Reverse index "KV block -> queries that selected it": one (key = head*blocks + block,
-//      value = token) pair per valid topk_idx entry, stable radix sort by key (tokens stay
-//      ascending inside a block), segment offsets by binary search.  No host round trips.
+//   1. Reverse index "KV block -> queries that selected it" as a stable counting sort of the valid
+//      topk_idx entries by (head, block), tokens ascending inside a block: per-tile block counts,
+//      prefix sums over tiles and over blocks, then a scatter that ranks the tokens of a 64-token
+//      group by bit masks.  Integer work only, no atomics whose order matters, no host round
+//      trips, no memsets: the whole backward can be recorded into a HIP graph.
 //   2. dK/dV: a workgroup keeps one KV block's K and V rows in registers (each wave owns 16
 //      keys) and streams the queries of that block two tokens at a time through LDS; per-chunk
 //      fp32 partials are reduced in a fixed order, so the result is deterministic (no atomics).
@@ -14,8 +16,6 @@
 //      runs only when the index phase is requested alone).
 #include <cstring>
 
-#include <rocprim/device/device_radix_sort.hpp>
-
 #include "retile.h"
 #include "delta.h"
 #include "dkdv.h"
@@ -23,9 +23,9 @@
 // ------------------------------------------------------------------------------------------
 // workspace carving (host and entry point must agree)
 struct BwdLayout {
-  size_t delta, cu_blk, keys_in, keys_out, vals_in, vals_out, seg_off, chunk_off, sort_tmp, kf, vf, partial, total;
-  size_t sort_tmp_bytes;
+  size_t delta, cu_blk, hist, queries, seg_off, chunk_off, kf, vf, partial, total;
   int64_t max_blocks, n_pairs, max_items, n_slots;
+  int tile_tokens, n_tiles;
 };
 
 static constexpr int LIST_CHUNK = 768;
@@ -37,6 +37,10 @@ constexpr int dkdv_block(int bs) { return bs >= 256 ? 64 : bs; }  // queries per
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// The counting sort walks the tokens in at most RI_MAX_TILES tiles (one wave each, 64 tokens at a time) and keeps the
+// counters of RI_CAP blocks in LDS at a time (more blocks: more sweeps over the tile).
+static constexpr int RI_MAX_TILES = 128, RI_CAP = 2048, RI_WAVES = 2;
+
 static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t topk, int64_t bs) {
   BwdLayout L;
   const int64_t ebs = dkdv_block((int)bs);
@@ -44,22 +48,16 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.n_pairs = Hkv * T * topk * (bs / ebs);
   const int chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
   L.max_items = (L.n_pairs + chunk - 1) / chunk + Hkv * L.max_blocks;
-  size_t tmp = 0;
-  uint32_t* nk = nullptr;
-  int32_t* nv = nullptr;
-  (void)rocprim::radix_sort_pairs(nullptr, tmp, nk, nk, nv, nv, (size_t)L.n_pairs, 0u, 32u, (hipStream_t)0);
-  L.sort_tmp_bytes = tmp;
+  L.tile_tokens = (int)(((T + RI_MAX_TILES - 1) / RI_MAX_TILES + 63) / 64 * 64);
+  L.n_tiles = (int)((T + L.tile_tokens - 1) / L.tile_tokens);
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += align256(bytes); return o; };
   L.delta = take((size_t)Hq * T * 4);
   L.cu_blk = take((size_t)(B + 1) * 4);
-  L.keys_in = take((size_t)L.n_pairs * 4);
-  L.keys_out = take((size_t)L.n_pairs * 4);
-  L.vals_in = take((size_t)L.n_pairs * 4);
-  L.vals_out = take((size_t)L.n_pairs * 4);
+  L.hist = take((size_t)Hkv * L.n_tiles * L.max_blocks * 4);   // [head][tile][block] counts, then their prefix over tiles
+  L.queries = take((size_t)L.n_pairs * 4);
   L.seg_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.chunk_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
-  L.sort_tmp = take(tmp);
   L.n_slots = nsa_chunk_slots(T, B);
   L.kf = take(retile_bytes(T, B, Hkv, D));   // row-fragment copies of K and V for the dQ pass
   L.vf = take(retile_bytes(T, B, Hkv, D));
@@ -74,39 +72,140 @@ __global__ __launch_bounds__(256) void seq_blocks_kernel(const int32_t* __restri
   block_count_prefix_256(cu, batch, bs, cu_blk);
 }
 
-__global__ __launch_bounds__(256) void emit_pairs_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ cu,
-                                                         const int32_t* __restrict__ cu_blk, int batch, int total_len, int Hkv,
-                                                         int topk, int bs, int ebs, int max_blocks, long long ish, long long isn,
-                                                         long long isk, uint32_t* __restrict__ keys, int32_t* __restrict__ vals) {
-  // one thread per (head, token, entry, piece of ebs keys inside the selected block); bs == ebs: one piece
-  const int sub = bs / ebs;
-  const long long n = (long long)Hkv * total_len * topk * sub;
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  const int s = (int)(i % sub);
-  const int e = (int)((i / sub) % topk);
-  const int t = (int)((i / ((long long)sub * topk)) % total_len);
-  const int h = (int)(i / ((long long)sub * topk * total_len));
-  const int b = find_sequence(cu, batch, t);
-  const int pos = t - cu[b];
-  const int blk = idx[(long long)h * ish + (long long)t * isn + (long long)e * isk];
-  const int piece = blk * sub + s;
-  const bool ok = blk >= 0 && blk <= pos / bs && piece * ebs <= pos;  // pieces wholly after the query hold nothing it sees
-  keys[i] = ok ? (uint32_t)(h * max_blocks + cu_blk[b] + piece) : (uint32_t)(Hkv * max_blocks);
-  vals[i] = t;
+struct RiParams {
+  const int32_t* idx; const int32_t* cu; const int32_t* cu_blk;
+  int batch, total_len, Hkv, topk, bs, ebs, max_blocks, tile_tokens, n_tiles;
+  long long ish, isn, isk;
+  int32_t* hist;            // [Hkv][n_tiles][max_blocks]: counts (written by the counting pass), then exclusive prefix over tiles
+  const int32_t* seg_off;   // scatter pass: first slot of every (head, block) segment
+  int32_t* queries;         // scatter pass: token ids, segment by segment, ascending inside a segment
+};
+
+// One wave per (head, tile of consecutive tokens), 64 tokens (one per lane) at a time.  Entry (token, e) is valid iff
+// 0 <= blk <= own block (and, for 256-key blocks split in four, the piece starts at or before the token).  The rank of
+// a token among the tokens of its group that selected the same block comes from a 64-bit mask per block (bit = lane),
+// built with LDS or-operations whose order cannot matter; the blocks' running counts within the tile sit next to the
+// masks.  SCATTER = false: writes the tile's count of every block.  SCATTER = true: writes every token to
+// seg_off[segment] + (entries of earlier tiles) + (entries of earlier groups of this tile) + rank.
+// A block listed twice by one token is counted and stored once.
+template <bool SCATTER>
+__global__ __launch_bounds__(64 * RI_WAVES) void reverse_index_kernel(RiParams p) {
+  __shared__ unsigned long long mask_s[RI_WAVES][RI_CAP];
+  __shared__ int cnt_s[RI_WAVES][RI_CAP];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int tile = blockIdx.x * RI_WAVES + wave, h = blockIdx.y;
+  if (tile >= p.n_tiles) return;   // waves never meet at a workgroup barrier
+  unsigned long long* mask = mask_s[wave];
+  int* cnt = cnt_s[wave];
+  const int sub = p.bs / p.ebs, n_e = p.topk * sub;
+  const int t_begin = tile * p.tile_tokens, t_end = min(p.total_len, t_begin + p.tile_tokens);
+  int32_t* hist = p.hist + ((long long)h * p.n_tiles + tile) * p.max_blocks;
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  for (int r0 = 0; r0 < p.max_blocks; r0 += RI_CAP) {
+    for (int i = lane; i < RI_CAP; i += 64) { mask[i] = 0ull; cnt[i] = 0; }
+    wave_sync();
+    for (int t0 = t_begin; t0 < t_end; t0 += 64) {
+      const int t = t0 + lane;
+      const bool live = t < t_end;
+      const int b = find_sequence(p.cu, p.batch, live ? t : t_begin);
+      const int pos = t - p.cu[b], first_blk = p.cu_blk[b] - r0;
+      const int32_t* ip = p.idx + (long long)h * p.ish + (long long)(live ? t : t_begin) * p.isn;
+      // block of entry i relative to r0, or -1 when the entry names nothing this token sees (or lies outside the sweep)
+      auto local_block = [&](int i) {
+        const int blk = ip[(long long)(i / sub) * p.isk];
+        const int piece = blk * sub + i % sub;
+        const bool ok = live && blk >= 0 && blk <= pos / p.bs && piece * p.ebs <= pos;
+        const int lb = first_blk + piece;
+        return ok && lb >= 0 && lb < RI_CAP ? lb : -1;
+      };
+      for (int i = 0; i < n_e; i++) {
+        const int lb = local_block(i);
+        if (lb >= 0) atomicOr(&mask[lb], 1ull << lane);
+      }
+      wave_sync();
+      if (SCATTER) {
+        for (int i = 0; i < n_e; i++) {
+          const int lb = local_block(i);
+          if (lb < 0) continue;
+          const int rank = __popcll(mask[lb] & ((1ull << lane) - 1ull));
+          p.queries[p.seg_off[h * p.max_blocks + r0 + lb] + hist[r0 + lb] + cnt[lb] + rank] = t;
+        }
+        wave_sync();
+      }
+      // the lowest lane of every mask adds the group's entries to the block's count and clears the mask
+      for (int i = 0; i < n_e; i++) {
+        const int lb = local_block(i);
+        if (lb < 0) continue;
+        const unsigned long long m = mask[lb];
+        if (m != 0ull && __builtin_ctzll(m) == lane) { cnt[lb] += __popcll(m); mask[lb] = 0ull; }
+      }
+      wave_sync();
+    }
+    if (!SCATTER)
+      for (int i = lane; i < min(RI_CAP, p.max_blocks - r0); i += 64) hist[r0 + i] = cnt[i];
+    wave_sync();
+  }
 }
 
-// seg_off[j] = first sorted position whose key >= j, j in [0, n_seg]; chunk counts alongside.
-__global__ __launch_bounds__(256) void segment_offsets_kernel(const uint32_t* __restrict__ keys, long long n, int n_seg,
-                                                              int32_t* __restrict__ seg_off) {
-  const int j = blockIdx.x * 256 + threadIdx.x;
-  if (j > n_seg) return;
-  long long lo = 0, hi = n;  // first position with keys[pos] >= j
-  while (lo < hi) {
-    long long mid = (lo + hi) >> 1;
-    if (keys[mid] < (uint32_t)j) lo = mid + 1; else hi = mid;
+// hist[h][tile][blk] -> exclusive prefix over the tiles; total[h * max_blocks + blk] = the sum.  A workgroup owns 64
+// segments (lanes, coalesced) and splits the tiles over its 4 waves: partial sums, then the prefixes.
+__global__ __launch_bounds__(256) void tile_prefix_kernel(int32_t* __restrict__ hist, int32_t* __restrict__ total, int Hkv, int n_tiles, int max_blocks) {
+  __shared__ int part[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int seg = blockIdx.x * 64 + lane, n_seg = Hkv * max_blocks;
+  const bool live = seg < n_seg;
+  const int h = live ? seg / max_blocks : 0, blk = live ? seg % max_blocks : 0;
+  int32_t* col = hist + (long long)h * n_tiles * max_blocks + blk;
+  const int per = (n_tiles + 3) / 4, c0 = min(n_tiles, wave * per), c1 = min(n_tiles, c0 + per);
+  int sum = 0;
+  if (live)
+    for (int c = c0; c < c1; c++) sum += col[(long long)c * max_blocks];
+  part[wave][lane] = sum;
+  __syncthreads();
+  int run = 0;
+  for (int w = 0; w < wave; w++) run += part[w][lane];
+  if (live) {
+    for (int c = c0; c < c1; c++) {
+      const int v = col[(long long)c * max_blocks];
+      col[(long long)c * max_blocks] = run;
+      run += v;
+    }
+    if (wave == 3) total[seg] = run;
   }
-  seg_off[j] = (int32_t)lo;
+}
+
+// seg_off = exclusive scan of total over the segments (seg_off[n_seg] = number of valid entries) and chunk_off =
+// exclusive scan of ceil(total / chunk): one workgroup, thread t owns a run of consecutive segments.  total may
+// alias chunk_off (every thread reads its run before anything is written).
+__global__ __launch_bounds__(1024) void segment_scan_kernel(const int32_t* total, int n_seg, int chunk, int32_t* __restrict__ seg_off,
+                                                            int32_t* chunk_off) {
+  __shared__ int part_a[1024], part_b[1024];
+  const int tid = threadIdx.x, per = (n_seg + 1023) / 1024;
+  const int j0 = min(n_seg, tid * per), j1 = min(n_seg, j0 + per);
+  int a = 0, b = 0;
+  for (int j = j0; j < j1; j++) { const int c = total[j]; a += c; b += (c + chunk - 1) / chunk; }
+  part_a[tid] = a; part_b[tid] = b;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int va = tid >= d ? part_a[tid - d] : 0, vb = tid >= d ? part_b[tid - d] : 0;
+    __syncthreads();
+    part_a[tid] += va; part_b[tid] += vb;
+    __syncthreads();
+  }
+  int ra = part_a[tid] - a, rb = part_b[tid] - b;
+  // the counts of this thread's run are read again here: nobody has written them yet (other threads write only
+  // their own runs of chunk_off, and seg_off is a different array)
+  for (int j = j0; j < j1; j++) {
+    const int c = total[j];
+    seg_off[j] = ra; chunk_off[j] = rb;
+    ra += c; rb += (c + chunk - 1) / chunk;
+  }
+  __syncthreads();
+  if (tid == 1023) { seg_off[n_seg] = part_a[1023]; chunk_off[n_seg] = part_b[1023]; }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -278,24 +377,20 @@ struct BwdArgs {
 static int build_reverse_index(const BwdArgs& a, const BwdLayout& L) {
   char* ws = a.ws;
   int32_t* cu_blk = (int32_t*)(ws + L.cu_blk);
-  uint32_t* keys_in = (uint32_t*)(ws + L.keys_in);
-  uint32_t* keys_out = (uint32_t*)(ws + L.keys_out);
-  int32_t* vals_in = (int32_t*)(ws + L.vals_in);
-  int32_t* vals_out = (int32_t*)(ws + L.vals_out);
   int32_t* seg_off = (int32_t*)(ws + L.seg_off);
   int32_t* chunk_off = (int32_t*)(ws + L.chunk_off);
   const int n_seg = (int)(a.Hkv * L.max_blocks);
-  seq_blocks_kernel<<<1, 256, 0, a.stream>>>(a.cu, (int)a.B, dkdv_block((int)a.bs), cu_blk);
-  emit_pairs_kernel<<<(unsigned)((L.n_pairs + 255) / 256), 256, 0, a.stream>>>(
-      a.idx, a.cu, cu_blk, (int)a.B, (int)a.T, (int)a.Hkv, (int)a.topk, (int)a.bs, dkdv_block((int)a.bs), (int)L.max_blocks, a.ish, a.isn, a.isk,
-      keys_in, vals_in);
-  unsigned bits = 1;
-  while ((1ull << bits) <= (unsigned long long)n_seg) bits++;
-  size_t tmp = L.sort_tmp_bytes;
-  if (rocprim::radix_sort_pairs(ws + L.sort_tmp, tmp, keys_in, keys_out, vals_in, vals_out, (size_t)L.n_pairs, 0u, bits, a.stream) != hipSuccess)
-    return NSA_ERR_LAUNCH;
-  segment_offsets_kernel<<<(n_seg + 1 + 255) / 256, 256, 0, a.stream>>>(keys_out, L.n_pairs, n_seg, seg_off);
-  chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_off, seg_off + 1, n_seg, chunk_off, dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK));
+  RiParams p;
+  p.idx = a.idx; p.cu = a.cu; p.cu_blk = cu_blk; p.batch = (int)a.B; p.total_len = (int)a.T; p.Hkv = (int)a.Hkv; p.topk = (int)a.topk;
+  p.bs = (int)a.bs; p.ebs = dkdv_block((int)a.bs); p.max_blocks = (int)L.max_blocks; p.tile_tokens = L.tile_tokens; p.n_tiles = L.n_tiles;
+  p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.hist = (int32_t*)(ws + L.hist); p.seg_off = seg_off; p.queries = (int32_t*)(ws + L.queries);
+  const dim3 grid((unsigned)((L.n_tiles + RI_WAVES - 1) / RI_WAVES), (unsigned)a.Hkv);
+  seq_blocks_kernel<<<1, 256, 0, a.stream>>>(a.cu, (int)a.B, p.ebs, cu_blk);
+  reverse_index_kernel<false><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
+  // the per-segment totals live in chunk_off until the scan replaces them
+  tile_prefix_kernel<<<(n_seg + 63) / 64, 256, 0, a.stream>>>(p.hist, chunk_off, (int)a.Hkv, L.n_tiles, (int)L.max_blocks);
+  segment_scan_kernel<<<1, 1024, 0, a.stream>>>(chunk_off, n_seg, dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK), seg_off, chunk_off);
+  reverse_index_kernel<true><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
   return nsa_check_launch();
 }
 
@@ -317,7 +412,7 @@ static int run_bwd(const BwdArgs& a) {
   }
   if (a.out_seg_off) {
     (void)hipMemcpyAsync(a.out_seg_off, ws + L.seg_off, (size_t)(n_seg + 1) * 4, hipMemcpyDeviceToDevice, a.stream);
-    (void)hipMemcpyAsync(a.out_queries, ws + L.vals_out, (size_t)L.n_pairs * 4, hipMemcpyDeviceToDevice, a.stream);
+    (void)hipMemcpyAsync(a.out_queries, ws + L.queries, (size_t)L.n_pairs * 4, hipMemcpyDeviceToDevice, a.stream);
   }
   // dQ first: it leaves delta behind for the dK/dV pass
   if (a.phases & NSA_BWD_PHASE_DQ) {
@@ -339,7 +434,7 @@ static int run_bwd(const BwdArgs& a) {
     DkdvParams p;
     p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.cu = a.cu;
     p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_begin = (const int32_t*)(ws + L.seg_off); p.seg_end = p.seg_begin + 1;
-    p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.vals_out);
+    p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.queries);
     p.partial = (float*)(ws + L.partial);
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
     p.qsn = (int)a.qsn; p.qsh = (int)a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = (int)a.dsn; p.dsh = (int)a.dsh;
@@ -393,7 +488,8 @@ extern "C" int nsa_topk_attn_bwd(const void* q, const void* k, const void* v, co
   if (!q || !k || !v || !o || !dout || !lse || !topk_idx || !cu_seqlens || !dq || !dk || !dv || !strides || !workspace) return NSA_ERR_BAD_ARG;
   if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
   if ((out_segment_offsets == nullptr) != (out_queries == nullptr)) return NSA_ERR_BAD_ARG;
-  if (num_kv_heads * total_len * topk >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
+  // 31-bit positions in the reverse index (256-key blocks are listed as four 64-key pieces)
+  if (num_kv_heads * total_len * topk * (block_size / dkdv_block((int)block_size)) >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
   for (int i = 0; i < 10; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;  // 16-byte loads, 31-bit strides
   for (int i = 13; i < 19; i++) if (strides[i] % 4 != 0) return NSA_ERR_UNSUPPORTED;      // 8-byte stores
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)dout) % 16 != 0) return NSA_ERR_UNSUPPORTED;

@@ -93,27 +93,82 @@ def test_backward_matches_oracle(device, lens, Hq, Hkv, d, bs, topk, dtype, loca
     _grad_check(device, lens, Hq, Hkv, d, bs, topk, dtype, local)
 
 
-def test_reverse_index_bit_exact_and_deterministic(device):
+def _expand_to_pieces(idx, cu, bs, piece):
+    """Ids of the `piece`-key pieces of the selected bs-key blocks that start at or before each token (-1 elsewhere)."""
+    sub = bs // piece
+    pos = torch.cat([torch.arange(int(b - a)) for a, b in zip(cu[:-1].tolist(), cu[1:].tolist())]).to(idx.device)
+    ids = idx[..., None].long() * sub + torch.arange(sub, device=idx.device)
+    ok = (idx[..., None] >= 0) & (idx[..., None] <= (pos // bs)[None, :, None, None]) & (ids * piece <= pos[None, :, None, None])
+    return torch.where(ok, ids, torch.full_like(ids, -1)).flatten(2).to(torch.int32)
+
+
+@pytest.mark.parametrize("lens,Hkv,bs,topk", [
+    ([700, 64, 1500], 2, 64, 6),
+    ([300, 5, 900, 257], 2, 256, 3),        # 256-key blocks are indexed as four 64-key pieces
+    ([70000, 100], 1, 32, 4),               # more blocks than the counting sort keeps in LDS at a time (two sweeps)
+    ([1], 3, 128, 2),
+])
+def test_reverse_index_bit_exact_and_deterministic(device, lens, Hkv, bs, topk):
     from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
-    lens, Hq, Hkv, d, bs, topk = [700, 64, 1500], 16, 2, 64, 64, 6
+    Hq, d = 4 * Hkv, 64
     q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device)
     idx = make_topk_idx(cu, bs, topk, Hkv, seed=4)
     o, lse = _topk_sparse_attention_fwd(q, k, v, idx, bs, cu, cu, None, None, d ** -0.5)
     do = torch.randn_like(o)
     dq, dk, dv, seg_off, queries = _topk_sparse_attention_bwd(
         o, do, lse, q, k, v, idx, bs, cu, cu, None, None, d ** -0.5, return_reverse_index=True)
-    cu_blk, offs, qs = oracle.build_reverse_index(idx.cpu().numpy(), cu.cpu().numpy(), bs)
+    ebs = 64 if bs == 256 else bs
+    want_idx = _expand_to_pieces(idx, cu, bs, ebs) if ebs != bs else idx
+    cu_blk, offs, qs = oracle.build_reverse_index(want_idx.cpu().numpy(), cu.cpu().numpy(), ebs)
     T, B = int(cu[-1]), len(lens)
-    max_blocks = T // bs + B
+    max_blocks = T // ebs + B
     seg_off, queries = seg_off.cpu().numpy(), queries.cpu().numpy()
     total_blocks = int(cu_blk[-1])
     for h in range(Hkv):
         for g in range(total_blocks):
             s = h * max_blocks + g
-            got = queries[seg_off[s]:seg_off[s + 1]].tolist()
-            assert got == qs[h, offs[h, g]:offs[h, g + 1]].tolist(), (h, g)
+            assert seg_off[s + 1] - seg_off[s] == offs[h, g + 1] - offs[h, g], (h, g)
+            assert (queries[seg_off[s]:seg_off[s + 1]] == qs[h, offs[h, g]:offs[h, g + 1]]).all(), (h, g)
         for g in range(total_blocks, max_blocks):                      # unused segments are empty
             s = h * max_blocks + g
             assert seg_off[s] == seg_off[s + 1]
     dq2, dk2, dv2 = _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, None, None, d ** -0.5)
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+
+
+def test_forward_backward_replayed_from_a_hip_graph(device):
+    """Forward + backward recorded once into a HIP graph (nothing in them allocates, synchronises or clears memory with
+    a memset) and replayed on fresh inputs, with eager work and synchronisation between the replays: every replay
+    must equal the eager result bit for bit."""
+    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
+    lens, Hq, Hkv, d, bs, topk = [900, 130, 2000], 32, 2, 128, 64, 8
+    q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device)
+    T = int(cu[-1])
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=1)
+    do = torch.randn_like(q)
+    sm = d ** -0.5
+
+    def step():
+        o, lse = _topk_sparse_attention_fwd(q, k, v, idx, bs, cu, cu, None, None, sm)
+        return (o,) + tuple(_topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, None, None, sm))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    g = torch.Generator(device=device).manual_seed(9)
+    for r in range(4):
+        for x in (q, k, v, do):
+            x.copy_(torch.randn(x.shape, generator=g, device=device).to(x.dtype))
+        idx.copy_(make_topk_idx(cu, bs, topk, Hkv, seed=10 + r))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in outs]
+        want = step()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("o", "dq", "dk", "dv"), got, want):
+            assert torch.equal(a, b), (name, r)
