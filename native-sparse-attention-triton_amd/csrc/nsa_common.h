@@ -228,6 +228,44 @@ __device__ __forceinline__ long long xcd_remap(long long wg, long long n_wg) {
   return (wg % 8) * per + wg / 8;
 }
 
+// How the two query-stationary kernels (one wave per (token, kv-head, head tile)) share their work items out over
+// the 8 XCDs.  Hardware hands workgroup i to XCD i % 8; a stream = the tokens of one (kv-head, head tile), whose
+// K/V should stay on as few L2s as possible.  When the streams divide the XCDs evenly and the batch is a single
+// sequence, each stream is cut into 8 / streams contiguous parts of equal estimated cost, one per XCD: a
+// token's cost grows with its position (its blocks are drawn from a longer prefix, of which the L2 holds a
+// smaller share); measured on single sequences of 16K..64K tokens the cost per token is proportional to
+// q0 + q, q = position / 64 and q0 = q0_l2_blocks x (the 64-key blocks of K and V that fit one XCD's 4 MiB L2), with
+// q0_l2_blocks about 5.5 for the forward and 8 for the dQ pass (more work per block at the same traffic).  With
+// equal token counts instead, the XCD holding the late half of a sequence ran 40 % longer than its partner.
+// parts = 0: every XCD takes an equal share of all items in (stream, token) order.
+struct XcdSchedule {
+  int parts;        // XCDs per stream, or 0
+  int wgs_per_xcd;  // workgroups (of 4 items) each XCD is given
+  int bound[9];     // part j of a stream holds the 64-token runs [bound[j], bound[j + 1])
+};
+static inline XcdSchedule nsa_xcd_schedule(long long total_len, long long batch, int streams, int head_dim, double q0_l2_blocks) {
+  XcdSchedule s;
+  s.parts = 0; s.wgs_per_xcd = 0;
+  for (int i = 0; i < 9; i++) s.bound[i] = 0;
+  const long long runs = (total_len + 63) / 64;
+  if (batch != 1 || streams <= 0 || streams > 8 || 8 % streams != 0 || runs < 64) return s;
+  const int parts = 8 / streams;
+  const double q0 = q0_l2_blocks * (4.0 * 1024 * 1024) / (64.0 * head_dim * 4), total = q0 * runs + 0.5 * runs * runs;
+  s.parts = parts;
+  s.bound[parts] = (int)runs;
+  long long longest = 0;
+  for (int j = 1; j <= parts; j++) {
+    if (j < parts) {
+      // C(q) = q0 q + q^2 / 2 = (j / parts) C(runs)
+      const double target = total * j / parts;
+      s.bound[j] = (int)(-q0 + __builtin_sqrt(q0 * q0 + 2.0 * target));
+    }
+    if (s.bound[j] - s.bound[j - 1] > longest) longest = s.bound[j] - s.bound[j - 1];
+  }
+  s.wgs_per_xcd = (int)(longest * 16);
+  return s;
+}
+
 static inline int nsa_check_launch() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? NSA_OK : NSA_ERR_LAUNCH;

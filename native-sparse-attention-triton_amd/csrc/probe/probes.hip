@@ -1,0 +1,135 @@
+// Memory-system and MFMA probes for the benchmark report (libnsa_probe.so; nothing in the operator library or the
+// Python package uses them).  Each one isolates a rate that bounds one of the attention kernels:
+//   nsa_probe_gather_blocks : the access pattern of the two query-stationary kernels without their arithmetic -
+//                             one wave per (token, kv-head) fetches the 64-key blocks named by topk_idx from the
+//                             fragment-major K / V copies, 32 KiB per block, and folds them into a checksum;
+//   nsa_probe_gather_rows   : the access pattern of the dK/dV pass - 4 KiB rows at random offsets of a buffer;
+//   nsa_probe_copy          : a plain copy (reference point for the FETCH_SIZE / WRITE_SIZE counters);
+//   nsa_probe_mfma          : back-to-back independent MFMAs on registers (the matrix-core ceiling).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void probe_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, long long n) {
+  // a workgroup moves 16 KiB per trip: four 16-byte pieces per thread, all loads before the stores
+  for (long long i = (long long)blockIdx.x * 1024 + threadIdx.x; i < n; i += (long long)gridDim.x * 1024) {
+    uint4 x[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) x[u] = i + 256 * u < n ? src[i + 256 * u] : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < 4; u++) if (i + 256 * u < n) dst[i + 256 * u] = x[u];
+  }
+}
+
+// kf / vf: [Hkv][n_slots][32 keys][D = 128] 2-byte elements, a 64-key block = 16 KiB of each; idx [Hkv][T][topk].
+// fold > 0: block ids are taken modulo fold (a working set that stays in L2).  contiguous_split = 1: the first half
+// of a head's tokens on one XCD, the second half on its partner (workgroup i runs on XCD i % 8).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void probe_gather_blocks_kernel(
+    const uint4* __restrict__ kf, const uint4* __restrict__ vf, const int32_t* __restrict__ idx, int T, int Hkv, int topk, int n_slots, int fold,
+    uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long long per = (gridDim.x + 7) / 8;
+  const long long item = ((blockIdx.x % 8) * per + blockIdx.x / 8) * 4 + wave;
+  if (item >= (long long)T * Hkv) return;
+  const int t = (int)(item % T), h = (int)(item / T);
+  const int32_t* ip = idx + ((long long)h * T + t) * topk;
+  // a 32-key slot = 32 x 128 x 2 B = 512 uint4; a 64-key block = two slots = 16 fragments of 64 lanes x 16 B, in K and in V
+  const uint4* kb = kf + (long long)h * n_slots * 512 + lane;
+  const uint4* vb = vf + (long long)h * n_slots * 512 + lane;
+  uint4 acc = {0u, 0u, 0u, 0u};
+  const int my_blk = lane < topk ? ip[lane] : -1;
+  unsigned long long todo = __ballot(my_blk >= 0);
+  while (todo) {
+    const int e = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    int blk = __builtin_amdgcn_readlane(my_blk, e);
+    if (fold > 0) blk %= fold;
+    const uint4* kp = kb + (long long)(2 * blk) * 512;
+    const uint4* vp = vb + (long long)(2 * blk) * 512;
+    uint4 x[32];
+#pragma unroll
+    for (int f = 0; f < 16; f++) { x[f] = kp[f * 64]; x[16 + f] = vp[f * 64]; }
+#pragma unroll
+    for (int f = 0; f < 32; f++) { acc.x ^= x[f].x; acc.y ^= x[f].y; acc.z ^= x[f].z; acc.w ^= x[f].w; }
+  }
+  out[item * 64 + lane] = acc;
+}
+
+// every wave reads `reads` (a multiple of 8) rows of 4 KiB at pseudo-random row indices of buf, eight rows in flight
+__global__ __launch_bounds__(256) void probe_gather_rows_kernel(const uint4* __restrict__ buf, long long n_rows, int reads, uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  unsigned long long state = 0x9E3779B97F4A7C15ull * (unsigned long long)(wave + 1);
+  uint4 acc = {0u, 0u, 0u, 0u};
+  for (int r = 0; r < reads; r += 8) {
+    uint4 x[32];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      state = state * 6364136223846793005ull + 1442695040888963407ull;
+      const long long row = (long long)((state >> 20) % (unsigned long long)n_rows);
+      const uint4* p = buf + row * 256 + lane;
+#pragma unroll
+      for (int c = 0; c < 4; c++) x[4 * u + c] = p[c * 64];
+    }
+#pragma unroll
+    for (int u = 0; u < 32; u++) { acc.x ^= x[u].x; acc.y ^= x[u].y; acc.z ^= x[u].z; acc.w ^= x[u].w; }
+  }
+  out[wave * 64 + lane] = acc;
+}
+
+template <int SHAPE>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, float* __restrict__ out) {
+  bf16x8 a, b;
+  for (int i = 0; i < 8; i++) { a[i] = (__bf16)(threadIdx.x * 0.001f + i); b[i] = (__bf16)(1.f - threadIdx.x * 0.002f); }
+  float sum = 0.f;
+  if (SHAPE == 16) {
+    f32x4 c[8];
+    for (int j = 0; j < 8; j++) c[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) c[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c[j], 0, 0, 0);
+    }
+    for (int j = 0; j < 8; j++) sum += c[j][0] + c[j][1] + c[j][2] + c[j][3];
+  } else {
+    f32x16 c[4];
+    for (int j = 0; j < 4; j++) for (int r = 0; r < 16; r++) c[j][r] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) c[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c[j], 0, 0, 0);
+    }
+    for (int j = 0; j < 4; j++) for (int r = 0; r < 16; r++) sum += c[j][r];
+  }
+  out[(long long)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+extern "C" int nsa_probe_copy(const void* src, void* dst, long long bytes, void* stream) {
+  probe_copy_kernel<<<16384, 256, 0, (hipStream_t)stream>>>((const uint4*)src, (uint4*)dst, bytes / 16);
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+extern "C" int nsa_probe_gather_blocks(const void* kf, const void* vf, const int32_t* idx, int total_len, int num_kv_heads, int topk,
+                                       int n_slots, int fold, void* out, void* stream) {
+  if (topk > 64) return -2;
+  long long n_wg = ((long long)total_len * num_kv_heads + 3) / 4;
+  n_wg = (n_wg + 7) / 8 * 8;
+  probe_gather_blocks_kernel<<<(unsigned)n_wg, 256, 0, (hipStream_t)stream>>>((const uint4*)kf, (const uint4*)vf, idx, total_len, num_kv_heads,
+                                                                               topk, n_slots, fold, (uint4*)out);
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+extern "C" int nsa_probe_gather_rows(const void* buf, long long n_rows, int row_bytes, int reads_per_wave, int n_workgroups, void* out, void* stream) {
+  if (row_bytes != 4096 || reads_per_wave % 8 != 0) return -2;
+  probe_gather_rows_kernel<<<n_workgroups, 256, 0, (hipStream_t)stream>>>((const uint4*)buf, n_rows, reads_per_wave, (uint4*)out);
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+// flops per launch = n_workgroups * 4 waves * iters * 8 (or 4) MFMAs * 16384 (or 32768) flops
+extern "C" int nsa_probe_mfma(int shape, int iters, int n_workgroups, float* out, void* stream) {
+  if (shape == 16) probe_mfma_kernel<16><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (shape == 32) probe_mfma_kernel<32><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else return -2;
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}

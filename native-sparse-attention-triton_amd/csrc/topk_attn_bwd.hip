@@ -217,6 +217,7 @@ struct DqParams {
   const int32_t* idx; const int32_t* cu; void* dq;
   int total_len, batch, Hkv, G, GT, topk, n_slots;
   long long n_items;
+  XcdSchedule sched;
   long long qsn, qsh, dsn, dsh, osn, osh, ish, isn, isk, dqsn, dqsh;
   float qk_scale, sm_scale;
 };
@@ -237,11 +238,19 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   // scalar wave index: token, sequence, block ids and fragment addresses are then computed once per wave
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, lg = lane >> 4;
-  const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
-  if (item >= p.n_items) return;
-  const int t = (int)(item % p.total_len);
-  const int gt = (int)((item / p.total_len) % p.GT);
-  const int h = (int)(item / ((long long)p.total_len * p.GT));
+  int t, gt, h;
+  if (p.sched.parts) {
+    const int xcd = blockIdx.x & 7, stream = xcd / p.sched.parts, part = xcd % p.sched.parts;
+    t = p.sched.bound[part] * 64 + (blockIdx.x >> 3) * 4 + wave;
+    if (t >= min(p.sched.bound[part + 1] * 64, p.total_len)) return;
+    h = stream / p.GT; gt = stream % p.GT;
+  } else {
+    const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
+    if (item >= p.n_items) return;
+    t = (int)(item % p.total_len);
+    gt = (int)((item / p.total_len) % p.GT);
+    h = (int)(item / ((long long)p.total_len * p.GT));
+  }
   const int b = find_sequence(p.cu, p.batch, t);
   const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
   const int pos = t - s0, qb = pos / BS;
@@ -427,7 +436,9 @@ static int run_bwd(const BwdArgs& a) {
     p.qsn = a.qsn; p.qsh = a.qsh; p.dsn = a.dsn; p.dsh = a.dsh; p.osn = a.osn; p.osh = a.osh;
     p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
+    p.sched = nsa_xcd_schedule(a.T, a.B, GT * (int)a.Hkv, (int)a.D, 8.0);
     long long n_wg = ((p.n_items + 3) / 4 + 7) / 8 * 8;
+    if (p.sched.parts) n_wg = 8ll * p.sched.wgs_per_xcd;
     dq_kernel<T, D, BS><<<(unsigned)n_wg, 256, 0, a.stream>>>(p);
   }
   if (a.phases & NSA_BWD_PHASE_DKDV) {

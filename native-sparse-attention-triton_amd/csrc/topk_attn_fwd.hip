@@ -14,6 +14,7 @@ struct TopkFwdParams {
   const void* q; const void* kf; const void* vf; const int32_t* idx; void* o; float* lse; const int32_t* cu;
   int total_len, batch, Hkv, G, GT, topk, n_slots;
   long long n_items;
+  XcdSchedule sched;
   long long qsn, qsh, ish, isn, isk, osn, osh;
   float qk_scale;  // sm_scale * log2(e)
 };
@@ -28,11 +29,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // fragment addresses) is computed once per wave on the scalar unit
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, lg = lane >> 4;
-  const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
-  if (item >= p.n_items) return;
-  const int t = (int)(item % p.total_len);
-  const int gt = (int)((item / p.total_len) % p.GT);
-  const int h = (int)(item / ((long long)p.total_len * p.GT));
+  int t, gt, h;
+  if (p.sched.parts) {
+    const int xcd = blockIdx.x & 7, stream = xcd / p.sched.parts, part = xcd % p.sched.parts;
+    t = p.sched.bound[part] * 64 + (blockIdx.x >> 3) * 4 + wave;
+    if (t >= min(p.sched.bound[part + 1] * 64, p.total_len)) return;
+    h = stream / p.GT; gt = stream % p.GT;
+  } else {
+    const long long item = xcd_remap(blockIdx.x, gridDim.x) * 4 + wave;
+    if (item >= p.n_items) return;
+    t = (int)(item % p.total_len);
+    gt = (int)((item / p.total_len) % p.GT);
+    h = (int)(item / ((long long)p.total_len * p.GT));
+  }
   const int b = find_sequence(p.cu, p.batch, t);
   const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
   const int pos = t - s0, qb = pos / BS;
@@ -172,6 +181,7 @@ static int launch_fwd(const TopkFwdParams& p, const void* k, long long ksn, long
   if (phases & NSA_FWD_PHASE_ATTEND) {
     long long n_wg = (p.n_items + 3) / 4;
     n_wg = (n_wg + 7) / 8 * 8;
+    if (p.sched.parts) n_wg = 8ll * p.sched.wgs_per_xcd;
     topk_fwd_kernel<T, D, BS><<<dim3((unsigned)n_wg), 256, 0, stream>>>(p);
   }
   return nsa_check_launch();
@@ -226,6 +236,7 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   p.total_len = (int)total_len; p.batch = (int)batch; p.Hkv = (int)num_kv_heads; p.G = (int)(num_q_heads / num_kv_heads);
   p.GT = (p.G + 15) / 16; p.topk = (int)topk; p.n_slots = (int)nsa_chunk_slots(total_len, batch);
   p.n_items = (long long)total_len * p.GT * p.Hkv;
+  p.sched = nsa_xcd_schedule(total_len, batch, p.GT * p.Hkv, (int)head_dim, 5.5);
   p.qsn = q_stride_n; p.qsh = q_stride_h;
   p.ish = idx_stride_h; p.isn = idx_stride_n; p.isk = idx_stride_k; p.osn = o_stride_n; p.osh = o_stride_h;
   p.qk_scale = sm_scale * NSA_LOG2E;
