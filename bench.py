@@ -356,6 +356,7 @@ def bench_probes(args, dev):
     pl.nsa_probe_copy.argtypes = [P, P, LL, P]
     pl.nsa_probe_gather_blocks.argtypes = [P, P, P, I, I, I, I, I, P, P]
     pl.nsa_probe_gather_rows.argtypes = [P, LL, I, I, I, P, P]
+    pl.nsa_probe_tile_gather.argtypes = [P, P, P, I, I, I, I, P, P, P]
     pl.nsa_probe_mfma.argtypes = [I, I, I, P, P]
     # block gather on the K / V fragment copies the forward left in its workspace
     _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_f)
@@ -372,6 +373,12 @@ def bench_probes(args, dev):
     for name, fold in (("gather_blocks_real_ids", 0), ("gather_blocks_folded_into_2MiB_per_head", 64)):
         ms = _time_ms(lambda: gather(fold), it, 1)
         probes[name] = {"ms": round(ms, 4), "TBps_into_the_CUs": round(n_blocks * 32768 / ms / 1e9, 2)}
+    if topk <= 32 and N <= 131072:
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        tile = lambda: pl.nsa_probe_tile_gather(ws_f.data_ptr(), ws_f.data_ptr() + copy_bytes, idx_c.data_ptr(), N, HKV, topk, n_slots,
+                                                sink.data_ptr(), flag.data_ptr(), st)
+        ms = _time_ms(tile, it, 1)
+        probes["gather_blocks_shared_in_24_token_tiles_through_LDS_ring"] = {"ms": round(ms, 4), "gave_up": int(flag.item())}
     # random 4 KiB rows: what the dK/dV pass asks of the memory system
     for name, mib in (("gather_rows_4KiB_in_1GiB", 1024), ("gather_rows_4KiB_in_128MiB", 128)):
         buf = torch.empty(mib << 20, dtype=torch.uint8, device=dev).random_()

@@ -53,20 +53,79 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(PoolParams p, T* __restri
   st16(y + (long long)n * p.ysn + (long long)h * p.ysh + 8 * c, out);
 }
 
+// Forward for launches large enough to be bound by bandwidth: the window of an output piece is split over SPLIT
+// threads of 16 rows each, whose 16 loads are all issued before the first is used (one round trip per thread
+// instead of kernel_size / 8 in a row, and SPLIT times as many threads in flight); the partial sums meet in LDS and
+// are added in window order.  Threads of a wave hold consecutive pieces of the same rows (coalesced).
+template <typename T, int D, int SPLIT>
+__global__ __launch_bounds__(256) void pool_fwd_split_kernel(PoolParams p, T* __restrict__ y) {
+  using v8 = typename Elem<T>::v8;
+  constexpr int C = D / 8, PPW = 256 / SPLIT;   // output pieces per workgroup
+  __shared__ float part[SPLIT > 1 ? SPLIT - 1 : 1][PPW][8];
+  const int sub = threadIdx.x / PPW, pl = threadIdx.x % PPW;
+  const long long i = (long long)blockIdx.x * PPW + pl;   // (n, h, c), c fastest
+  const bool live = i < (long long)p.total_y * p.H * C;
+  const int c = (int)(i % C), h = (int)((i / C) % p.H), n = live ? (int)(i / ((long long)C * p.H)) : 0;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (live) {
+    const int b = find_sequence(p.ycu, p.batch, n);
+    const int row0 = p.cu[b] + (n - p.ycu[b]) * p.st + 16 * sub;
+    const T* xp = (const T*)p.x + (long long)row0 * p.xsn + (long long)h * p.xsh + 8 * c;
+    v8 xv[16];
+#pragma unroll
+    for (int u = 0; u < 16; u++) xv[u] = ld16<v8>(xp + (long long)u * p.xsn);
+    float wk[16];
+    if (p.w) {
+      const T* wp = (const T*)p.w + (long long)h * p.wsh + 16 * sub;
+#pragma unroll
+      for (int u = 0; u < 16; u++) wk[u] = (float)wp[u];
+    } else {
+#pragma unroll
+      for (int u = 0; u < 16; u++) wk[u] = 1.f / (float)p.ks;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(wk[u], (float)xv[u][j], acc[j]);
+  }
+  if (SPLIT > 1) {
+    if (sub > 0) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) part[sub - 1][pl][j] = acc[j];
+    }
+    __syncthreads();
+    if (sub > 0) return;
+#pragma unroll
+    for (int s2 = 1; s2 < SPLIT; s2++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc[j] += part[s2 - 1][pl][j];
+  }
+  if (!live) return;
+  v8 out;
+#pragma unroll
+  for (int j = 0; j < 8; j++) out[j] = (T)acc[j];
+  st16(y + (long long)n * p.ysn + (long long)h * p.ysh + 8 * c, out);
+}
+
 template <typename T, int D>
 __global__ __launch_bounds__(256) void pool_dx_kernel(PoolParams p, const T* __restrict__ dy, long long dysn, long long dysh,
                                                       T* __restrict__ dx, long long dxsn, long long dxsh) {
   using v8 = typename Elem<T>::v8;
   constexpr int C = D / 8;
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // (t, h, c)
-  if (i >= (long long)p.total_x * p.H * C) return;
-  const int c = (int)(i % C), h = (int)((i / C) % p.H), t = (int)(i / ((long long)C * p.H));
-  const int b = find_sequence(p.cu, p.batch, t);
+  // a workgroup owns 256 / C consecutive tokens of one head; the sequence of its first token is found once (scalar),
+  // a thread whose token lies beyond that sequence's end searches on its own
+  constexpr int TPB = 256 / C;
+  const int c = threadIdx.x % C, t = blockIdx.x * TPB + threadIdx.x / C, h = blockIdx.y;
+  if (threadIdx.x / C >= TPB || t >= p.total_x) return;
+  int b = find_sequence(p.cu, p.batch, blockIdx.x * TPB);
+  if (t >= p.cu[b + 1]) b = find_sequence(p.cu, p.batch, t);
   const int pos = t - p.cu[b];
   const int ylen = p.ycu[b + 1] - p.ycu[b];
+  // windows n with n * st <= pos <= n * st + ks - 1; a power-of-two stride divides by a shift
+  const int sh = (p.st & (p.st - 1)) == 0 ? __builtin_ctz(p.st) : -1;
   int n_lo = pos - p.ks + 1;
-  n_lo = n_lo <= 0 ? 0 : (n_lo + p.st - 1) / p.st;
-  int n_hi = pos / p.st;
+  n_lo = n_lo <= 0 ? 0 : (sh >= 0 ? (n_lo + p.st - 1) >> sh : (n_lo + p.st - 1) / p.st);
+  int n_hi = sh >= 0 ? pos >> sh : pos / p.st;
   n_hi = n_hi < ylen - 1 ? n_hi : ylen - 1;
   const T* wp = p.w ? (const T*)p.w + (long long)h * p.wsh : nullptr;
   const float wavg = 1.f / (float)p.ks;
@@ -143,14 +202,22 @@ __global__ __launch_bounds__(64) void pool_dw_final_kernel(const float* __restri
 template <typename T, int D>
 static int pool_fwd_t(const PoolParams& p, void* y, hipStream_t s) {
   const long long n = (long long)p.total_y * p.H * (D / 8);
-  if (n > 0) pool_fwd_kernel<T, D><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p, (T*)y);
+  if (n <= 0) return NSA_OK;
+  // big launches: one round of loads per thread; small ones (a decode step pools one window per sequence) keep the
+  // plain kernel, whose summation order the single-launch decode preparation reproduces bit for bit
+  const bool big = n >= 32768;
+  if (big && p.ks == 16) pool_fwd_split_kernel<T, D, 1><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p, (T*)y);
+  else if (big && p.ks == 32) pool_fwd_split_kernel<T, D, 2><<<(unsigned)((n + 127) / 128), 256, 0, s>>>(p, (T*)y);
+  else if (big && p.ks == 64) pool_fwd_split_kernel<T, D, 4><<<(unsigned)((n + 63) / 64), 256, 0, s>>>(p, (T*)y);
+  else if (big && p.ks == 128) pool_fwd_split_kernel<T, D, 8><<<(unsigned)((n + 31) / 32), 256, 0, s>>>(p, (T*)y);
+  else pool_fwd_kernel<T, D><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p, (T*)y);
   return nsa_check_launch();
 }
 template <typename T, int D>
 static int pool_bwd_t(const PoolParams& p, const void* dy, long long dysn, long long dysh, void* dx, long long dxsn, long long dxsh,
                       void* dw, long long dwsh, float* partial, hipStream_t s) {
-  const long long n = (long long)p.total_x * p.H * (D / 8);
-  pool_dx_kernel<T, D><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p, (const T*)dy, dysn, dysh, (T*)dx, dxsn, dxsh);
+  constexpr int TPB = 256 / (D / 8);
+  pool_dx_kernel<T, D><<<dim3((unsigned)((p.total_x + TPB - 1) / TPB), (unsigned)p.H), 256, 0, s>>>(p, (const T*)dy, dysn, dysh, (T*)dx, dxsn, dxsh);
   if (dw) {
     const int n_tiles = (p.total_y + DW_TILE - 1) / DW_TILE;
     if (n_tiles > 0) pool_dw_partial_kernel<T, D><<<dim3((unsigned)n_tiles, (unsigned)p.H), 256, 0, s>>>(p, (const T*)dy, dysn, dysh, partial, n_tiles);

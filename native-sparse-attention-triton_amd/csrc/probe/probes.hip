@@ -133,3 +133,140 @@ extern "C" int nsa_probe_mfma(int shape, int iters, int n_workgroups, float* out
   else return -2;
   return hipGetLastError() == hipSuccess ? 0 : -4;
 }
+
+// ------------------------------------------------------------------------------------------
+// nsa_probe_tile_gather: the block gather with sharing inside a tile of 24 consecutive tokens.  A workgroup of 8
+// waves (3 tokens each) forms the ascending list of the distinct blocks its tokens selected, stages each block once
+// in a ring of 4 LDS buffers (asynchronous global->LDS copies issued by whichever wave reaches a safe point
+// first), and every wave reads the staged block once per token of its own that selected it.  No arithmetic:
+// the time is what the memory system and the ring allow a forward kernel of this shape.
+struct TileCtl { int pos[8]; int ready[4]; int next_issue; int n_list; int err; int wave_cnt[8]; };
+
+__global__ __launch_bounds__(512) void probe_tile_gather_kernel(const uint4* __restrict__ kf, const uint4* __restrict__ vf, const int32_t* __restrict__ idx,
+                                                                int T, int Hkv, int topk, int n_slots, int n_tiles, uint4* __restrict__ out,
+                                                                int* __restrict__ err_out) {
+  constexpr int NW = 8, TPW = 3, TT = NW * TPW, R = 4, NB_MAX = 2048, L_MAX = TT * 32;
+  __shared__ __attribute__((aligned(1024))) uint4 ring[R][2048];   // 32 KiB per block: 16 K fragments then 16 V fragments of 64 x 16 B
+  __shared__ unsigned bmask[NB_MAX];
+  __shared__ unsigned short list_blk[L_MAX];
+  __shared__ unsigned list_mask[L_MAX];
+  __shared__ TileCtl ctl;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const long long per = (gridDim.x + 7) / 8;
+  const long long item = (blockIdx.x % 8) * per + blockIdx.x / 8;    // consecutive tiles of a head on one XCD
+  if (item >= (long long)n_tiles * Hkv) return;
+  const int h = (int)(item / n_tiles), tile = (int)(item % n_tiles);
+  const int t0 = tile * TT, nt = min(TT, T - t0);
+  const int nb = (t0 + nt - 1) / 64 + 1;
+  for (int i = tid; i < nb; i += 512) bmask[i] = 0u;
+  if (tid < NW) ctl.pos[tid] = 0;
+  if (tid < R) ctl.ready[tid] = 0;
+  if (tid == 0) { ctl.next_issue = 0; ctl.err = 0; }
+  __syncthreads();
+  for (int e = tid; e < TT * topk; e += 512) {
+    const int tk = e / topk, k = e % topk;
+    if (tk < nt) {
+      const int blk = idx[((long long)h * T + t0 + tk) * topk + k];
+      if (blk >= 0 && blk <= (t0 + tk) / 64) atomicOr(&bmask[blk], 1u << tk);
+    }
+  }
+  __syncthreads();
+  int base = 0;
+  for (int c0 = 0; c0 < nb; c0 += 512) {
+    const int blk = c0 + tid;
+    const unsigned m = blk < nb ? bmask[blk] : 0u;
+    const unsigned long long ball = __ballot(m != 0u);
+    if (lane == 0) ctl.wave_cnt[wave] = __popcll(ball);
+    __syncthreads();
+    int off = base, total = 0;
+    for (int w = 0; w < NW; w++) { const int c = ctl.wave_cnt[w]; if (w < wave) off += c; total += c; }
+    off += __popcll(ball & ((1ull << lane) - 1ull));
+    if (m != 0u) { list_blk[off] = (unsigned short)blk; list_mask[off] = m; }
+    __syncthreads();
+    base += total;
+  }
+  const int n_list = base;
+  const uint4* kb = kf + (long long)h * n_slots * 512 + lane;
+  const uint4* vb = vf + (long long)h * n_slots * 512 + lane;
+  uint4 acc[TPW];
+  for (int j = 0; j < TPW; j++) acc[j] = uint4{0u, 0u, 0u, 0u};
+  int pending = -1;
+  // publish a finished copy, then start the next one if its buffer is free and nobody else has claimed it
+  auto produce = [&]() {
+    if (pending >= 0) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the copy has landed in LDS
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      if (lane == 0) __hip_atomic_store(&ctl.ready[pending % R], pending + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      pending = -1;
+    }
+    const int j = __hip_atomic_load(&ctl.next_issue, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (j >= n_list) return;
+    int lo = 1 << 30;
+    for (int w = 0; w < NW; w++) lo = min(lo, __hip_atomic_load(&ctl.pos[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+    if (lo + R <= j) return;          // some wave still needs the block that sits in this buffer
+    int won = 0;
+    if (lane == 0) {
+      int expect = j;
+      won = __hip_atomic_compare_exchange_strong(&ctl.next_issue, &expect, j + 1, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    won = __builtin_amdgcn_readfirstlane(won);
+    if (!won) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const int blk = list_blk[j];
+    const uint4* kp = kb + (long long)(2 * blk) * 512;
+    const uint4* vp = vb + (long long)(2 * blk) * 512;
+    unsigned char* dst = (unsigned char*)&ring[j % R][0];
+#pragma unroll
+    for (int f = 0; f < 16; f++) {
+      __builtin_amdgcn_global_load_lds(kp + f * 64, (__attribute__((address_space(3))) void*)(dst + f * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(vp + f * 64, (__attribute__((address_space(3))) void*)(dst + 16384 + f * 1024), 16, 0, 0);
+    }
+    pending = j;
+  };
+  for (int i = 0; i < n_list; i++) {
+    const unsigned m = (list_mask[i] >> (TPW * wave)) & ((1u << TPW) - 1u);
+    if (m != 0u) {
+      int spins = 0;
+      while (__hip_atomic_load(&ctl.ready[i % R], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != i + 1) {
+        produce();
+        __builtin_amdgcn_s_sleep(1);
+        if (++spins > (1 << 22) || __hip_atomic_load(&ctl.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
+          if (lane == 0) { __hip_atomic_store(&ctl.err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); *err_out = 1; }
+          i = n_list;   // give up: every wave leaves its loop
+          break;
+        }
+      }
+      if (i >= n_list) break;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      const uint4* src = &ring[i % R][lane];
+#pragma unroll
+      for (int j = 0; j < TPW; j++) {
+        if (m & (1u << j)) {
+          uint4 x[32];
+#pragma unroll
+          for (int f = 0; f < 32; f++) x[f] = src[f * 64];
+#pragma unroll
+          for (int f = 0; f < 32; f++) { acc[j].x ^= x[f].x; acc[j].y ^= x[f].y; acc[j].z ^= x[f].z; acc[j].w ^= x[f].w; }
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (lane == 0) __hip_atomic_store(&ctl.pos[wave], i + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    produce();
+  }
+  // a copy this wave started may still be in flight: let it land before the workgroup's LDS is given away
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  if (pending >= 0 && lane == 0) __hip_atomic_store(&ctl.ready[pending % R], pending + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  for (int j = 0; j < TPW; j++)
+    if (wave * TPW + j < nt) out[((long long)h * T + t0 + wave * TPW + j) * 64 + lane] = acc[j];
+}
+
+extern "C" int nsa_probe_tile_gather(const void* kf, const void* vf, const int32_t* idx, int total_len, int num_kv_heads, int topk, int n_slots,
+                                     void* out, int* err_out, void* stream) {
+  if (topk > 32 || (total_len + 63) / 64 > 2048) return -2;
+  const int n_tiles = (total_len + 23) / 24;
+  long long n_wg = ((long long)n_tiles * num_kv_heads + 7) / 8 * 8;
+  probe_tile_gather_kernel<<<(unsigned)n_wg, 512, 0, (hipStream_t)stream>>>((const uint4*)kf, (const uint4*)vf, idx, total_len, num_kv_heads, topk,
+                                                                            n_slots, n_tiles, (uint4*)out, err_out);
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}
