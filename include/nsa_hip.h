@@ -10,7 +10,7 @@
  *  - dtype: NSA_BF16 or NSA_FP16 for q/k/v/x/w/o tensors; accumulation is fp32.
  *  - Strides are in elements; the innermost (head_dim) stride must be 1.
  *  - Varlen tensors are [total_len, heads, head_dim]; cu_seqlens is int32 [batch+1].
- *  - sm_scale of the prefill/training attention entry points must be positive (NSA_ERR_UNSUPPORTED otherwise).
+ *  - sm_scale may be any finite number (NSA_ERR_BAD_ARG for NaN or infinity).
  *  - Return value: NSA_OK (0) or a negative NSA_ERR_* code; nothing is launched on error.
  *  - Re-entrant: no global state (one exception, stated there: nsa_topk_decode_static).
  */

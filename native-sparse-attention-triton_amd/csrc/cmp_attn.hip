@@ -154,7 +154,13 @@ __global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams 
     const T* qp = (const T*)p.q + (long long)(ti.s0q + (pos < ti.lq ? pos : 0)) * p.qsn + (long long)hh * p.qsh + 8 * lg;
 #pragma unroll
     for (int kk = 0; kk < NK; kk++) qf[j][kk] = live ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+    // running maxima are taken on unscaled scores: a negative scale is applied as -q and |scale|
+    if (p.qk_scale < 0.f) {
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) qf[j][kk] = negated16(qf[j][kk]);
+    }
   }
+  const float qs = fabsf(p.qk_scale);
   int tile_lo, tile_hi, unused;
   visible_range(min(ti.i0 + 15, ti.lq - 1), ti.lq, ti.lk, p.ks, p.st, p.window, unused, tile_hi);
   visible_range(ti.i0, ti.lq, ti.lk, p.ks, p.st, p.window, tile_lo, unused);
@@ -220,16 +226,16 @@ __global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams 
       // the reference maximum only moves when a chunk beats it by more than RESCALE_SLACK in the exponent:
       // until then probabilities are formed against the old reference (at most 2^RESCALE_SLACK: exact in
       // the fp32 sums, within range of bf16/fp16) and alpha stays exactly 1, so the rescale below is skipped
-      const float m_new = (mloc - m[j]) * p.qk_scale > RESCALE_SLACK ? mloc : m[j];
-      alpha[j] = fast_exp2((m[j] - m_new) * p.qk_scale);
-      const float mb = m_new * p.qk_scale;
+      const float m_new = (mloc - m[j]) * qs > RESCALE_SLACK ? mloc : m[j];
+      alpha[j] = fast_exp2((m[j] - m_new) * qs);
+      const float mb = m_new * qs;
       m[j] = m_new;
       float psum = 0.f;
 #pragma unroll
       for (int sub = 0; sub < 2; sub++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float x = fast_exp2(__builtin_fmaf(s[j][sub][r], p.qk_scale, -mb));
+          const float x = fast_exp2(__builtin_fmaf(s[j][sub][r], qs, -mb));
           psum += x;
           pf[j][4 * sub + r] = (T)x;
         }
@@ -300,7 +306,7 @@ __global__ __launch_bounds__(64 * (16 / FWD_TPW)) void cmp_fwd_kernel(CmpParams 
         for (int r = 0; r < 4; r++) out[r] = (T)(acc[j][dt][r] * inv);
         st8(op + 16 * dt, out);
       }
-      if (lg == 0) p.lse[(long long)hh * p.total_q + ti.s0q + pos] = lt > 0.f ? m[j] * p.qk_scale + fast_log2(lt) : -INFINITY;
+      if (lg == 0) p.lse[(long long)hh * p.total_q + ti.s0q + pos] = lt > 0.f ? m[j] * qs + fast_log2(lt) : -INFINITY;
     }
   }
 }
@@ -781,14 +787,15 @@ static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, c
                       int dtype, void* stream) {
   if (!q || !k || !cu_q || !cu_k || !strides || Tq <= 0 || Tk < 0 || B <= 0 || Hkv <= 0 || Hq % Hkv != 0 || ks <= 0 || st <= 0) return NSA_ERR_BAD_ARG;
   if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
-  if (!(sm_scale > 0.f)) return NSA_ERR_UNSUPPORTED;  // running maxima are taken on unscaled scores
+  if (!(sm_scale == sm_scale) || sm_scale - sm_scale != 0.f) return NSA_ERR_BAD_ARG;  // NaN or infinite scale
   for (int i = 0; i < 6; i++) if (strides[i] % 8 != 0 || strides[i] >= (1ll << 31)) return NSA_ERR_UNSUPPORTED;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) % 16 != 0) return NSA_ERR_UNSUPPORTED;
   CmpParams& p = a.p;
   p.q = q; p.k = k; p.v = v; p.cu_q = cu_q; p.cu_k = cu_k; p.total_q = (int)Tq; p.batch = (int)B; p.Hkv = (int)Hkv;
   p.G = (int)(Hq / Hkv); p.GT = (p.G + 15) / 16; p.ks = (int)ks; p.st = (int)st;
   p.qsn = strides[0]; p.qsh = strides[1]; p.ksn = strides[2]; p.ksh = strides[3]; p.vsn = strides[4]; p.vsh = strides[5];
-  p.qk_scale = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale; p.window = -1;
+  // forward: a zero scale is applied as the smallest positive one (masked scores are -inf there, and 0 * inf has no value)
+  p.qk_scale = (sm_scale == 0.f ? 1.17549435e-38f : sm_scale) * NSA_LOG2E; p.sm_scale = sm_scale; p.window = -1;
   p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr; p.delta_out = nullptr;
   a.Tq = Tq; a.Tk = Tk; a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.stream = (hipStream_t)stream; a.ws = nullptr;
   return NSA_OK;

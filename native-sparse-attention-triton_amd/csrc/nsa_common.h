@@ -54,6 +54,12 @@ template <typename V> __device__ __forceinline__ V zero16() {
   uint4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(V, z);
 }
+// the eight 2-byte floating-point elements of a fragment with their signs flipped
+template <typename V> __device__ __forceinline__ V negated16(V v) {
+  uint4 r = __builtin_bit_cast(uint4, v);
+  r.x ^= 0x80008000u; r.y ^= 0x80008000u; r.z ^= 0x80008000u; r.w ^= 0x80008000u;
+  return __builtin_bit_cast(V, r);
+}
 template <typename V> __device__ __forceinline__ void st16(void* p, V v) {
   *reinterpret_cast<uint4*>(p) = __builtin_bit_cast(uint4, v);
 }

@@ -53,6 +53,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   v8 qf[NK];
 #pragma unroll
   for (int kk = 0; kk < NK; kk++) qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+  // Running maxima are taken on unscaled scores, which is only right for a positive scale: with a negative one the
+  // kernel works on -q and |scale| (the same products; a zero scale needs nothing: every probability is then 1).
+  const float qs = fabsf(p.qk_scale);
+  if (p.qk_scale < 0.f) {
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) qf[kk] = negated16(qf[kk]);
+  }
 
   f32x4 acc[NDT];
 #pragma unroll
@@ -122,22 +129,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       // RESCALE_SLACK in the exponent: until then probabilities are formed against the old reference
       // (at most 2^RESCALE_SLACK, exact in fp32 sums and within range of bf16/fp16), and the
       // accumulator rescale, a multiply per accumulator register, is skipped.
-      const bool moved = (mloc - m) * p.qk_scale > RESCALE_SLACK;
+      const bool moved = (mloc - m) * qs > RESCALE_SLACK;
       if (__ballot(moved)) {
         const float m_new = moved ? mloc : m;
-        const float alpha = fast_exp2((m - m_new) * p.qk_scale);
+        const float alpha = fast_exp2((m - m_new) * qs);
         m = m_new;
         lsum *= alpha;
 #pragma unroll
         for (int i = 0; i < NDT; i++) acc[i] *= alpha;
       }
-      const float mb = m * p.qk_scale;
+      const float mb = m * qs;
       float psum = 0.f;
 #pragma unroll
       for (int nt = 0; nt < NS; nt++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float x = fast_exp2(__builtin_fmaf(s[nt][r], p.qk_scale, -mb));
+          const float x = fast_exp2(__builtin_fmaf(s[nt][r], qs, -mb));
           s[nt][r] = x;
           psum += x;
         }
@@ -167,7 +174,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int r = 0; r < 4; r++) out[r] = (T)(acc[dt][r] * inv);
       st8(op + 16 * dt, out);
     }
-    if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + t] = lsum > 0.f ? m * p.qk_scale + fast_log2(lsum) : -INFINITY;
+    if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + t] = lsum > 0.f ? m * qs + fast_log2(lsum) : -INFINITY;
   }
 }
 
@@ -225,7 +232,7 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   if (!q || !k || !v || !topk_idx || !o || !lse || !cu_seqlens || !workspace) return NSA_ERR_BAD_ARG;
   if (total_len <= 0 || batch <= 0 || num_kv_heads <= 0 || topk <= 0 || num_q_heads % num_kv_heads != 0) return NSA_ERR_BAD_ARG;
   if (total_len >= (1ll << 31)) return NSA_ERR_BAD_ARG;
-  if (!(sm_scale > 0.f)) return NSA_ERR_UNSUPPORTED;  // running maxima are taken on unscaled scores
+  if (!(sm_scale == sm_scale) || sm_scale - sm_scale != 0.f) return NSA_ERR_BAD_ARG;  // NaN or infinite scale
   // 16-byte fragment loads need 8-element alignment of every row start
   if ((q_stride_n | q_stride_h | k_stride_n | k_stride_h | v_stride_n | v_stride_h) % 8 != 0) return NSA_ERR_UNSUPPORTED;
   if ((o_stride_n | o_stride_h) % 4 != 0) return NSA_ERR_UNSUPPORTED;
@@ -239,7 +246,9 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   p.sched = nsa_xcd_schedule(total_len, batch, p.GT * p.Hkv, (int)head_dim, 5.5);
   p.qsn = q_stride_n; p.qsh = q_stride_h;
   p.ish = idx_stride_h; p.isn = idx_stride_n; p.isk = idx_stride_k; p.osn = o_stride_n; p.osh = o_stride_h;
-  p.qk_scale = sm_scale * NSA_LOG2E;
+  // a zero scale is applied as the smallest positive one: finite scores then still give probability 1, masked
+  // (-inf) scores still probability 0 (with an exact zero they would give 0 * inf)
+  p.qk_scale = (sm_scale == 0.f ? 1.17549435e-38f : sm_scale) * NSA_LOG2E;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, k, k_stride_n, k_stride_h, v, v_stride_n, v_stride_h, phases, s);
   if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, k, k_stride_n, k_stride_h, v, v_stride_n, v_stride_h, phases, s);

@@ -21,6 +21,11 @@ class NSADecodeGraph:
     selected, which makes the block ids independent of the longest sequence in the batch).  The cache must have
     been filled by a prefill of the same batch before the first `step`; a later prefill of another batch of the same
     size into the same cache can reuse the object.  Replays run on the stream that is current when `step` is called.
+
+    A recorded step cannot look at lengths on the host, so the object counts its replays since the last prefill and
+    raises once the longest sequence would outgrow the cache (`max_prompt_len + steps > cache.max_length`).  The
+    kernels themselves never write past a slab either: a sequence that has filled its rows is left as it is
+    (no token stored, length not advanced), which keeps memory safe but would make later outputs meaningless.
     """
 
     def __init__(self, cu_seqlens: torch.Tensor, num_q_heads: int, rope, cache, compress_weight: Tuple[torch.Tensor, torch.Tensor],
@@ -31,7 +36,7 @@ class NSADecodeGraph:
         batch = cu_seqlens.shape[0] - 1
         dev, dt = cache.sparse_kv_cache.device, cache.dtype
         self.cache = cache
-        self.max_steps_hint = cache.max_length
+        self._steps, self._prefill_serial = 0, cache.prefill_serial
         self.query = torch.zeros(batch, num_q_heads, cache.head_dim, dtype=dt, device=dev)
         self.key = torch.zeros(batch, cache.num_kv_heads, cache.head_dim, dtype=dt, device=dev)
         self.value = torch.zeros_like(self.key)
@@ -45,9 +50,18 @@ class NSADecodeGraph:
                                  compress_func, intra_block_pe, kernel_size, kernel_stride, block_size, topk, init_blocks,
                                  local_blocks, window_size)
 
+    def _count_step(self):
+        if self._prefill_serial != self.cache.prefill_serial:   # a new batch has been prefilled into the cache
+            self._steps, self._prefill_serial = 0, self.cache.prefill_serial
+        self._steps += 1
+        if self.cache.max_prompt_len + self._steps > self.cache.max_length:
+            raise RuntimeError("decode step %d of a %d-token prompt does not fit the cache (max_length %d)"
+                               % (self._steps, self.cache.max_prompt_len, self.cache.max_length))
+
     @torch.no_grad()
     def step(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, gate_value: torch.Tensor) -> torch.Tensor:
         """One new token per sequence; returns a view of the graph's output buffer (valid until the next call)."""
+        self._count_step()
         dst, src = [self.query, self.key, self.value, self.gate], [query, key, value, gate_value]
         if hasattr(torch, "_foreach_copy_"):
             torch._foreach_copy_(dst, src)   # one launch for the four copies
@@ -61,5 +75,6 @@ class NSADecodeGraph:
     def replay(self) -> torch.Tensor:
         """The same step for a caller that has already written the new token's states into `self.query`, `self.key`,
         `self.value` and `self.gate` (for example as the `out=` of its projections): no copies, one graph launch."""
+        self._count_step()
         self.graph.replay()
         return self.out

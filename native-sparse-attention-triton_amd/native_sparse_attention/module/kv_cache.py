@@ -74,6 +74,7 @@ class NSACache:
         self.dtype, self.device = dtype, device
         self.max_comp_length = (max_length - kernel_size) // kernel_stride + 1
         self.max_prompt_len = 0  # host copy of the longest prompt of the current batch (set at prefill)
+        self.prefill_serial = 0  # counts prefills: a recorded decode step restarts its step count when this changes
         self._staging_cu = None
         self._staging_out_cu = None
         self.static_shapes = False  # decode steps use the full slab extents instead of the current length bound
@@ -177,6 +178,7 @@ class NSACache:
         if step == 0:
             seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
             self.max_prompt_len = int(seqlens.max())  # the one host read of a prefill
+            self.prefill_serial += 1
             assert self.max_prompt_len <= self.max_length
             _, comp_cu = get_compressed_seqlens(cu_seqlens, self.kernel_size, self.kernel_stride)
             self._fill(self.compress_kv_cache, self.compress_kv_len, compress_key, compress_value, comp_cu,

@@ -45,10 +45,10 @@ def test_bad_arguments_are_rejected_without_launching():
 def test_more_host_side_checks():
     lib = _lib.load()
     fake = 1 << 20  # non-null, 16-byte aligned; never dereferenced: the checks below fail before any launch
-    # non-positive softmax scale is refused by the training/prefill attention entry points
+    # a softmax scale that is not a finite number is refused (any finite one, negative or zero included, is accepted)
     rc = lib.nsa_topk_attn_fwd(fake, fake, fake, fake, fake, fake, fake, 128, 1, 16, 1, 128, 4, 64, 2048, 128, 128, 128, 128, 128,
-                               512, 4, 1, 2048, 128, -0.1, 0, fake, 1 << 30, 3, None)
-    assert rc == -2
+                               512, 4, 1, 2048, 128, float("nan"), 0, fake, 1 << 30, 3, None)
+    assert rc == -1
     # the split of the linear_compress forward: cfg1 shape (1021 outputs, 4 heads, kernel 32, d 128) -> 16 splits of fp32 partials
     assert lib.nsa_linear_compress_fwd_workspace_bytes(1021, 3, 4, 128, 32) == 16 * 1021 * 4 * 128 * 4
     assert lib.nsa_linear_compress_fwd_workspace_bytes(200000, 1, 8, 128, 32) == 0          # enough workgroups already

@@ -96,3 +96,14 @@ def test_selection_is_reproducible_on_near_ties(device):
         noise = noise @ noise.T / 4096          # unrelated work between the calls
         _, again = compressed_attention(q, ck, cv, ks, st, bs, topk, cu, cuk)
         assert torch.equal(first, again)
+
+
+def test_negative_softmax_scale(device):
+    q, ck, cv, cu, cuk = _inputs([300, 200], 8, 2, 64, 32, 16, torch.bfloat16, device)
+    q = (q.float() * 0.3).bfloat16()
+    o, idx = compressed_attention(q, ck, cv, 32, 16, 64, 4, cu, cuk, 300, 17, -0.125)
+    want, want_idx, bscore = oracle.compressed_attention(q.float(), ck.float(), cv.float(), 32, 16, 64, 4, cu, cuk, 300, 17, -0.125,
+                                                         return_scores=True)
+    assert_close(o, want, "o")
+    qb = torch.cat([torch.arange(L, device=device) for L in (300, 200)]) // 64
+    assert_ids_match(idx, want_idx, bscore, qb, "topk_idx", min_overlap=0.9)

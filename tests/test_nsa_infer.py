@@ -210,3 +210,35 @@ def test_single_launch_prepare_equals_separate_operators(device, weighted, with_
             assert torch.equal(getattr(caches[0], slab)[:, b, :n], getattr(caches[1], slab)[:, b, :n]), (slab, b)
         n = min(int(caches[1].sliding_kv_len[b]), W)
         assert torch.equal(caches[0].sliding_kv_cache[:, b, :n], caches[1].sliding_kv_cache[:, b, :n]), ("ring", b)
+
+
+def test_graphed_decode_refuses_to_outgrow_the_cache(device):
+    """A recorded step cannot check lengths on the host: the graph object counts its replays and raises before the
+    longest sequence would need a row the cache does not have; a new prefill restarts the count."""
+    from native_sparse_attention.infer import NSADecodeGraph
+    from native_sparse_attention.module import RopeConfig, RotaryEmbedding
+    Hq, Hkv, d, ks, st, bs, topk, W = 16, 2, 128, 32, 16, 64, 4, 64
+    lens = [70, 33]
+    g = torch.Generator(device=device).manual_seed(3)
+    cu = cu_from_lens(lens, device)
+    T = int(cu[-1])
+    rope = RotaryEmbedding(RopeConfig(head_dim=d), device=device)
+    wk = torch.softmax(torch.randn(Hkv, ks, generator=g, device=device), -1).bfloat16()
+
+    def rnd(*shape):
+        return torch.randn(*shape, generator=g, device=device).bfloat16()
+
+    cache = NSACache(2, max(lens) + 3, Hkv, d, ks, st, W, torch.bfloat16, device)
+    tail = ((wk, wk), (weightedpool_compress, weightedpool_compress), None, ks, st, bs, topk, 1, 2, W)
+    prefill = lambda: nsa_infer(cu, 0, rnd(T, Hq, d), rnd(T, Hkv, d), rnd(T, Hkv, d), torch.sigmoid(rnd(T, Hq, 3).float()).bfloat16(), rope, cache, *tail)
+    prefill()
+    graph = NSADecodeGraph(cu, Hq, rope, cache, *tail)
+    tok = lambda: (rnd(2, Hq, d), rnd(2, Hkv, d), rnd(2, Hkv, d), torch.sigmoid(rnd(2, Hq, 3).float()).bfloat16())
+    for _ in range(3):
+        graph.step(*tok())
+    with pytest.raises(RuntimeError):
+        graph.step(*tok())
+    assert int(cache.sparse_kv_len[0]) == 73          # the refused step touched nothing
+    prefill()
+    graph.step(*tok())                                 # the count restarted with the new prompt
+    assert int(cache.sparse_kv_len[0]) == 71

@@ -172,3 +172,22 @@ def test_forward_backward_replayed_from_a_hip_graph(device):
         torch.cuda.synchronize()
         for name, a, b in zip(("o", "dq", "dk", "dv"), got, want):
             assert torch.equal(a, b), (name, r)
+
+
+@pytest.mark.parametrize("scale", [-0.2, 0.0, 3.0])
+def test_any_finite_softmax_scale(device, scale):
+    """The reference accepts any softmax scale (ops/triton/topk_sparse_attention.py:1133-1134 only fills in a default)."""
+    lens, Hq, Hkv, d, bs, topk = [300, 77], 16, 2, 64, 64, 4
+    q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device)
+    q, k = (q.float() * 0.5).bfloat16(), (k.float() * 0.5).bfloat16()
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=2)
+    q1, k1, v1 = (x.clone().requires_grad_() for x in (q, k, v))
+    o = topk_sparse_attention(q1, k1, v1, idx, bs, cu, scale)
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, k, v))
+    want = oracle.topk_sparse_attention(qf, kf, vf, idx, bs, cu, scale)
+    assert_close(o, want, "o")
+    do = torch.randn_like(o)
+    o.backward(do)
+    want.backward(do.float())
+    for name, a, b in (("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)):
+        assert_close(a, b, name, rel_to=max(1.0, b.abs().max().item()))
