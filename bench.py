@@ -22,6 +22,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "native-sparse-attention-triton_amd"))
 
 PEAK_BF16_TFLOPS = 2500.0        # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0           # MI355X HBM3E
 HQ, HKV, D, BS = 64, 4, 128, 64
 # reference-published Triton timings for this exact workload (its README.md:219,229): H100 fwd + bwd, ms
 H100_FWD_BWD_MS = 12.417 + 15.154
@@ -73,6 +74,16 @@ def cpu_baseline():
     }
 
 
+def _mfma_roofline(ops, whole_tflops):
+    """roofline object for a workload made of several operators: ops = [(name, ms, algorithmic FLOPs)]; the entry is the
+    MFMA-bound operator that takes the most time."""
+    rows = [{"kernel": n, "ms": ms, "algorithmic_flops": f, "tflops": f / ms / 1e9 if f else None,
+             "frac": f / ms / 1e9 / PEAK_BF16_TFLOPS if f else None} for n, ms, f in ops]
+    dom = max((r for r in rows if r["algorithmic_flops"]), key=lambda r: r["ms"])
+    return {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+            "frac": dom["frac"], "traffic": None, "step_frac": whole_tflops / PEAK_BF16_TFLOPS, "kernels": rows}
+
+
 def _time_ms(fn, iters, warm=2):
     for _ in range(warm):
         fn()
@@ -117,7 +128,13 @@ def bench_pipeline(args, dev):
     f_lin = 2 * 2.0 * int(cuk[-1]) * ks * D * D * HKV
     f_cmp = 4.0 * D * HQ * pairs
     f_top = 4.0 * D * bs * (HQ // HKV) * int((idx >= 0).sum())
+    ops = [("linear_compress (K and V: lin_fwd_kernel + lin_reduce_kernel)", t_lin, f_lin),
+           ("compressed_attention forward (cmp_fwd_kernel)", t_cmp, f_cmp),
+           ("block selection (cmp_select_kernel; recomputes the scores: no algorithmic FLOPs of its own)", t_sel, 0.0),
+           ("topk_sparse_attention forward (retile_kernel x2 + topk_fwd_kernel)", t_top, f_top)]
+    roof = _mfma_roofline(ops, (f_lin + f_cmp + f_top) / t_all / 1e9)
     return {
+        "roofline": roof,
         "metric": "NSA op pipeline forward ms (linear_compress x2 + compressed_attention w/ selection + topk_sparse_attention)",
         "value": t_all, "unit": "ms", "n_gpus": 1, "steps": it, "warmup": 2, "ms_per_step": t_all, "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -164,7 +181,15 @@ def bench_compressed(args, dev):
     pairs = sum((i - ks + 1) // st + 1 for i in range(ks - 1, N))
     f_fwd = 4.0 * D * Hq * pairs
     pool_bytes = (N * Hkv * D + 4095 * Hkv * D) * 2
+    ops = [("compressed_attention forward (cmp_fwd_kernel)", t_fwd, f_fwd),
+           ("block selection (cmp_select_kernel; recomputes the scores: no algorithmic FLOPs of its own)", t_sel, 0.0),
+           ("compressed_attention backward (dkdv_kernel over query ranges + dkdv_reduce_kernel + cmp_dq_kernel)", t_bwd, 2.5 * f_fwd)]
+    roof = _mfma_roofline(ops, 3.5 * f_fwd / t_all / 1e9)
+    roof["hbm_kernels"] = [{"kernel": "weightedpool forward, one tensor (pool_fwd_split_kernel; wrapper time, includes the length bookkeeping launch)",
+                            "ms": t_pool, "algorithmic_bytes": pool_bytes, "GBps": pool_bytes / t_pool / 1e6, "peak": PEAK_HBM_GBPS,
+                            "frac": pool_bytes / t_pool / 1e6 / PEAK_HBM_GBPS}]
     return {
+        "roofline": roof,
         "metric": "weightedpool + compressed_attention fwd+bwd ms (N=65536)", "value": t_all, "unit": "ms", "n_gpus": 1, "steps": it,
         "warmup": 1, "ms_per_step": t_all, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
@@ -246,7 +271,16 @@ def bench_decode(args, dev):
         t_w = _time_ms(lambda: flash_attention_decode(qd, cache.sliding_kv_cache[0, :B], cache.sliding_kv_cache[1, :B], wl), 20)
     key_rows = int(cache.compress_kv_len[:B].sum()) + 64 * int((idx >= 0).sum()) // Hkv + B * W
     alg_bytes = 2 * Hkv * D * 2 * key_rows
+    step_bytes = alg_bytes + 2 * B * (Hq + 2 * Hkv) * D * 2 + B * Hq * 3 * 2       # keys and values read + q, k, v, gate in and the output
+    roof = {"bound": "hbm", "kernel": "whole decode step (5 dependent launches, replayed from a HIP graph)", "achieved": step_bytes / us / 1e3,
+            "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": step_bytes / us / 1e3 / PEAK_HBM_GBPS, "traffic": None, "algorithmic_bytes": step_bytes,
+            "note": "a decode step moves a few MiB: it is bound by the latency of its dependent launches, not by bandwidth",
+            "kernels": [{"kernel": n, "us": t * 1e3, "GBps": bts / t / 1e6} for n, t, bts in (
+                ("compressed_attention_decode (decode_partial_kernel + decode_score_select_kernel)", t_c, 2 * Hkv * D * 2 * int(cache.compress_kv_len[:B].sum())),
+                ("topk_sparse_attention_decode (decode_partial_kernel + decode_merge_kernel)", t_s, 2 * Hkv * D * 2 * 64 * int((idx >= 0).sum()) // Hkv),
+                ("flash_attention_decode over the window (decode_partial_kernel + decode_merge_kernel)", t_w, 2 * Hkv * D * 2 * B * W))]}
     return {
+        "roofline": roof,
         "metric": "NSA decode step latency (us, cache update + compression + rope + three branches + gate), B=4, cached lens 2K..8K", "value": us, "unit": "us", "n_gpus": 1, "steps": steps,
         "warmup": 2, "ms_per_step": us / 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",

@@ -37,9 +37,9 @@ constexpr int dkdv_block(int bs) { return bs >= 256 ? 64 : bs; }  // queries per
 
 static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// The counting sort walks the tokens in at most RI_MAX_TILES tiles (one wave each, 64 tokens at a time) and keeps the
-// counters of RI_CAP blocks in LDS at a time (more blocks: more sweeps over the tile).
-static constexpr int RI_MAX_TILES = 128, RI_CAP = 2048, RI_WAVES = 2;
+// The counting sort walks the tokens in at most RI_MAX_TILES tiles (one wave each, 64 tokens at a time), keeps the
+// counters of RI_CAP blocks in LDS at a time (more blocks: more sweeps over the tile) and loads RI_ROW ids of a token at once.
+static constexpr int RI_MAX_TILES = 512, RI_CAP = 2048, RI_WAVES = 2, RI_ROW = 16;
 
 static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t topk, int64_t bs) {
   BwdLayout L;
@@ -87,8 +87,11 @@ struct RiParams {
 // built with LDS or-operations whose order cannot matter; the blocks' running counts within the tile sit next to the
 // masks.  SCATTER = false: writes the tile's count of every block.  SCATTER = true: writes every token to
 // seg_off[segment] + (entries of earlier tiles) + (entries of earlier groups of this tile) + rank.
-// A block listed twice by one token is counted and stored once.
-template <bool SCATTER>
+// A block listed twice by one token is counted and stored once.  SUB: pieces per selected block (1, or 4 for
+// 256-key blocks).  Everything a wave waits for from global memory is asked for in batches (the ids of 16
+// entries, then the offsets of all their segments): with one load per entry the kernel was a chain of a
+// few hundred dependent round trips.
+template <bool SCATTER, int SUB>
 __global__ __launch_bounds__(64 * RI_WAVES) void reverse_index_kernel(RiParams p) {
   __shared__ unsigned long long mask_s[RI_WAVES][RI_CAP];
   __shared__ int cnt_s[RI_WAVES][RI_CAP];
@@ -97,84 +100,117 @@ __global__ __launch_bounds__(64 * RI_WAVES) void reverse_index_kernel(RiParams p
   if (tile >= p.n_tiles) return;   // waves never meet at a workgroup barrier
   unsigned long long* mask = mask_s[wave];
   int* cnt = cnt_s[wave];
-  const int sub = p.bs / p.ebs, n_e = p.topk * sub;
+  constexpr int NE = RI_ROW * SUB;
   const int t_begin = tile * p.tile_tokens, t_end = min(p.total_len, t_begin + p.tile_tokens);
   int32_t* hist = p.hist + ((long long)h * p.n_tiles + tile) * p.max_blocks;
+  const int32_t* seg_off = SCATTER ? p.seg_off + (long long)h * p.max_blocks : nullptr;
   auto wave_sync = [] {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
+  // sequence of the tile's first token, found once; lanes beyond its end search on their own
+  const int b_first = find_sequence(p.cu, p.batch, t_begin);
+  const int end_first = p.cu[b_first + 1];
   for (int r0 = 0; r0 < p.max_blocks; r0 += RI_CAP) {
-    for (int i = lane; i < RI_CAP; i += 64) { mask[i] = 0ull; cnt[i] = 0; }
+    const int n_here = min(RI_CAP, p.max_blocks - r0);
+    for (int i = lane; i < n_here; i += 64) { mask[i] = 0ull; cnt[i] = 0; }
     wave_sync();
     for (int t0 = t_begin; t0 < t_end; t0 += 64) {
       const int t = t0 + lane;
       const bool live = t < t_end;
-      const int b = find_sequence(p.cu, p.batch, live ? t : t_begin);
-      const int pos = t - p.cu[b], first_blk = p.cu_blk[b] - r0;
-      const int32_t* ip = p.idx + (long long)h * p.ish + (long long)(live ? t : t_begin) * p.isn;
-      // block of entry i relative to r0, or -1 when the entry names nothing this token sees (or lies outside the sweep)
-      auto local_block = [&](int i) {
-        const int blk = ip[(long long)(i / sub) * p.isk];
-        const int piece = blk * sub + i % sub;
-        const bool ok = live && blk >= 0 && blk <= pos / p.bs && piece * p.ebs <= pos;
-        const int lb = first_blk + piece;
-        return ok && lb >= 0 && lb < RI_CAP ? lb : -1;
+      const int tt = live ? t : t_begin;
+      const int b = tt < end_first ? b_first : find_sequence(p.cu, p.batch, tt);
+      const int pos = tt - p.cu[b], first_blk = p.cu_blk[b] - r0, own = pos / p.bs;
+      const int32_t* ip = p.idx + (long long)h * p.ish + (long long)tt * p.isn;
+      // local block (relative to r0) of every (entry, piece) of a stretch of RI_ROW entries, -1 where it names
+      // nothing this token sees or lies outside the sweep
+      auto stretch = [&](int e0, int (&lb)[NE]) {
+        int row[RI_ROW];
+#pragma unroll
+        for (int j = 0; j < RI_ROW; j++) row[j] = e0 + j < p.topk ? ip[(long long)(e0 + j) * p.isk] : -1;
+#pragma unroll
+        for (int j = 0; j < RI_ROW; j++)
+#pragma unroll
+          for (int s2 = 0; s2 < SUB; s2++) {
+            const int blk = row[j], piece = blk * SUB + s2;
+            const bool ok = live && blk >= 0 && blk <= own && piece * p.ebs <= pos;
+            const int x = first_blk + piece;
+            lb[j * SUB + s2] = ok && x >= 0 && x < RI_CAP ? x : -1;
+          }
       };
-      for (int i = 0; i < n_e; i++) {
-        const int lb = local_block(i);
-        if (lb >= 0) atomicOr(&mask[lb], 1ull << lane);
+      // Three passes over the token's entries (mark, store, count), each complete before the next starts: the
+      // rank of a token must count every lower lane that names the block, at whatever entry position.
+      for (int e0 = 0; e0 < p.topk; e0 += RI_ROW) {
+        int lb[NE];
+        stretch(e0, lb);
+#pragma unroll
+        for (int i = 0; i < NE; i++)
+          if (lb[i] >= 0) atomicOr(&mask[lb[i]], 1ull << lane);
       }
       wave_sync();
       if (SCATTER) {
-        for (int i = 0; i < n_e; i++) {
-          const int lb = local_block(i);
-          if (lb < 0) continue;
-          const int rank = __popcll(mask[lb] & ((1ull << lane) - 1ull));
-          p.queries[p.seg_off[h * p.max_blocks + r0 + lb] + hist[r0 + lb] + cnt[lb] + rank] = t;
+        for (int e0 = 0; e0 < p.topk; e0 += RI_ROW) {
+          int lb[NE], base[NE];
+          stretch(e0, lb);
+#pragma unroll
+          for (int i = 0; i < NE; i++) {   // all offsets first (independent loads), then the stores
+            const int g = r0 + (lb[i] >= 0 ? lb[i] : 0);
+            base[i] = seg_off[g] + hist[g];
+          }
+#pragma unroll
+          for (int i = 0; i < NE; i++)
+            if (lb[i] >= 0) p.queries[base[i] + cnt[lb[i]] + __popcll(mask[lb[i]] & ((1ull << lane) - 1ull))] = t;
         }
         wave_sync();
       }
       // the lowest lane of every mask adds the group's entries to the block's count and clears the mask
-      for (int i = 0; i < n_e; i++) {
-        const int lb = local_block(i);
-        if (lb < 0) continue;
-        const unsigned long long m = mask[lb];
-        if (m != 0ull && __builtin_ctzll(m) == lane) { cnt[lb] += __popcll(m); mask[lb] = 0ull; }
+      for (int e0 = 0; e0 < p.topk; e0 += RI_ROW) {
+        int lb[NE];
+        stretch(e0, lb);
+#pragma unroll
+        for (int i = 0; i < NE; i++) {
+          if (lb[i] < 0) continue;
+          const unsigned long long m = mask[lb[i]];
+          if (m != 0ull && __builtin_ctzll(m) == lane) { cnt[lb[i]] += __popcll(m); mask[lb[i]] = 0ull; }
+        }
       }
       wave_sync();
     }
     if (!SCATTER)
-      for (int i = lane; i < min(RI_CAP, p.max_blocks - r0); i += 64) hist[r0 + i] = cnt[i];
+      for (int i = lane; i < n_here; i += 64) hist[r0 + i] = cnt[i];
     wave_sync();
   }
 }
 
 // hist[h][tile][blk] -> exclusive prefix over the tiles; total[h * max_blocks + blk] = the sum.  A workgroup owns 64
-// segments (lanes, coalesced) and splits the tiles over its 4 waves: partial sums, then the prefixes.
-__global__ __launch_bounds__(256) void tile_prefix_kernel(int32_t* __restrict__ hist, int32_t* __restrict__ total, int Hkv, int n_tiles, int max_blocks) {
-  __shared__ int part[4][64];
+// segments (lanes, coalesced) and splits the tiles over its 16 waves: partial sums, then the prefixes.
+__global__ __launch_bounds__(1024) void tile_prefix_kernel(int32_t* __restrict__ hist, int32_t* __restrict__ total, int Hkv, int n_tiles, int max_blocks) {
+  constexpr int NW = 16;
+  __shared__ int part[NW][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seg = blockIdx.x * 64 + lane, n_seg = Hkv * max_blocks;
   const bool live = seg < n_seg;
   const int h = live ? seg / max_blocks : 0, blk = live ? seg % max_blocks : 0;
   int32_t* col = hist + (long long)h * n_tiles * max_blocks + blk;
-  const int per = (n_tiles + 3) / 4, c0 = min(n_tiles, wave * per), c1 = min(n_tiles, c0 + per);
+  const int per = (n_tiles + NW - 1) / NW, c0 = min(n_tiles, wave * per), c1 = min(n_tiles, c0 + per);
   int sum = 0;
-  if (live)
+  if (live) {
+#pragma unroll 8
     for (int c = c0; c < c1; c++) sum += col[(long long)c * max_blocks];
+  }
   part[wave][lane] = sum;
   __syncthreads();
   int run = 0;
   for (int w = 0; w < wave; w++) run += part[w][lane];
   if (live) {
+#pragma unroll 8
     for (int c = c0; c < c1; c++) {
       const int v = col[(long long)c * max_blocks];
       col[(long long)c * max_blocks] = run;
       run += v;
     }
-    if (wave == 3) total[seg] = run;
+    if (wave == NW - 1) total[seg] = run;
   }
 }
 
@@ -395,11 +431,13 @@ static int build_reverse_index(const BwdArgs& a, const BwdLayout& L) {
   p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.hist = (int32_t*)(ws + L.hist); p.seg_off = seg_off; p.queries = (int32_t*)(ws + L.queries);
   const dim3 grid((unsigned)((L.n_tiles + RI_WAVES - 1) / RI_WAVES), (unsigned)a.Hkv);
   seq_blocks_kernel<<<1, 256, 0, a.stream>>>(a.cu, (int)a.B, p.ebs, cu_blk);
-  reverse_index_kernel<false><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
+  if (p.bs == p.ebs) reverse_index_kernel<false, 1><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
+  else reverse_index_kernel<false, 4><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
   // the per-segment totals live in chunk_off until the scan replaces them
-  tile_prefix_kernel<<<(n_seg + 63) / 64, 256, 0, a.stream>>>(p.hist, chunk_off, (int)a.Hkv, L.n_tiles, (int)L.max_blocks);
+  tile_prefix_kernel<<<(n_seg + 63) / 64, 1024, 0, a.stream>>>(p.hist, chunk_off, (int)a.Hkv, L.n_tiles, (int)L.max_blocks);
   segment_scan_kernel<<<1, 1024, 0, a.stream>>>(chunk_off, n_seg, dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK), seg_off, chunk_off);
-  reverse_index_kernel<true><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
+  if (p.bs == p.ebs) reverse_index_kernel<true, 1><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
+  else reverse_index_kernel<true, 4><<<grid, 64 * RI_WAVES, 0, a.stream>>>(p);
   return nsa_check_launch();
 }
 

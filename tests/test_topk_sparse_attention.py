@@ -107,6 +107,7 @@ def _expand_to_pieces(idx, cu, bs, piece):
     ([300, 5, 900, 257], 2, 256, 3),        # 256-key blocks are indexed as four 64-key pieces
     ([70000, 100], 1, 32, 4),               # more blocks than the counting sort keeps in LDS at a time (two sweeps)
     ([1], 3, 128, 2),
+    ([2500, 333], 1, 32, 20),               # more entries per token than the sort loads at a time
 ])
 def test_reverse_index_bit_exact_and_deterministic(device, lens, Hkv, bs, topk):
     from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
