@@ -384,6 +384,27 @@ def bench_probes(args, dev):
     parts["tokens_first_half_only"] = kernels_ms(rows(0, N // 2))
     parts["tokens_second_half_only"] = kernels_ms(rows(N // 2, N))
 
+    # Emulation of a key-range split over the XCDs of a head: kv-head 2h + p = kv-head h restricted to the selected blocks of
+    # parity p (q, k, v duplicated), so that every XCD owns one (head, parity) stream of all tokens and its L2 caches half the blocks.
+    # What a split forward / dQ pass would take before it merged its partial outputs.
+    def parity(pp):
+        x = torch.where((idx >= 0) & (idx % 2 == pp), idx, torch.full_like(idx, 1 << 30)).sort(-1).values
+        return torch.where(x == (1 << 30), torch.full_like(x, -1), x)
+    idx2 = torch.stack([parity(0), parity(1)], 1).reshape(2 * HKV, N, topk).contiguous()
+    k2, v2 = k.repeat_interleave(2, 1).contiguous(), v.repeat_interleave(2, 1).contiguous()
+    q2 = q.view(N, HKV, 1, HQ // HKV, D).expand(N, HKV, 2, HQ // HKV, D).reshape(N, 2 * HQ, D).contiguous()
+    do2 = do.view(N, HKV, 1, HQ // HKV, D).expand(N, HKV, 2, HQ // HKV, D).reshape(N, 2 * HQ, D).contiguous()
+    ws_f2 = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, 2 * HKV, D), dev)
+    ws_b2 = _lib.workspace(lib.nsa_topk_attn_bwd_workspace_bytes(N, 1, 2 * HQ, 2 * HKV, D, topk, BS), dev)
+    o2, lse2 = _topk_sparse_attention_fwd(q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_f2)
+    g2 = _topk_sparse_attention_bwd(o2, do2, lse2, q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_b2)
+    parts["block_parity_split_over_the_two_xcds_of_a_head_emulated"] = {
+        "pairs": int((idx2 >= 0).sum()),
+        "topk_fwd_kernel": round(_time_ms(lambda: _topk_sparse_attention_fwd(q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_f2, phases=2, out=(o2, lse2)), it, 1), 4),
+        "dq_kernel": round(_time_ms(lambda: _topk_sparse_attention_bwd(o2, do2, lse2, q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_b2, phases=4, out=g2), it, 1), 4),
+        "dkdv_kernel": None}
+    del q2, do2, k2, v2, o2, lse2, g2, ws_f2, ws_b2, idx2
+
     pl = ctypes.CDLL(os.path.join(os.path.dirname(_lib.lib_path()), "libnsa_probe.so"))
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P, LL, I = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
