@@ -114,7 +114,8 @@ int nsa_pool_bwd(const void* x, const void* w, const void* dy, void* dx, void* d
 /* ---- linear_compress ----------------------------------------------------------------------------
  * Forward: replaces linear_compress_fwd_kernel (native_sparse_attention/ops/triton/linear_compress.py:27-136,
  * launched at :379-410).  x [total_x,H,D]; w [H, kernel_size*D, D] contiguous; y [total_y,H,D].
- * workspace (16-byte aligned; may be NULL when the size query returns 0): fp32 partials of the split contraction.
+ * The forward adds the shares of its waves in LDS and needs no workspace: the size query returns 0 and the
+ * workspace arguments are ignored (both stay so that existing callers keep working).
  */
 size_t nsa_linear_compress_fwd_workspace_bytes(int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim, int64_t kernel_size);
 int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,

@@ -1,7 +1,7 @@
 // linear_compress: per-head sliding-window linear projection of K or V,
 //   y[n,h,:] = concat_k( x[s0 + n*stride + k, h, :] ) @ W[h]          W[h]: [kernel*D, D]
 // as strided-window GEMMs on the matrix cores, without materialising the unfolded windows.
-//   forward : Y^T[e][n]  = sum_{k,d} W[(k,d)][e] * Xwin[n][(k,d)]   W tiles staged in LDS, read transposed
+//   forward : Y^T[e][n]  = sum_{k,d} W[(k,d)][e] * Xwin[n][(k,d)]   W pieces transposed in registers, no LDS staging
 //   dX      : tokens grouped by phase (pos mod stride) share the same slices of W:
 //             dX^T[d][m] = sum_{j,e} W[(phase + j*stride, d)][e] * dY[m - j][e]   all operands straight from global
 //   dW      : dW^T[e][(k,d)] = sum_n dY[n][e] * x[row(n)+k][d]      both tiles through LDS, read transposed
@@ -13,7 +13,6 @@ struct LinParams {
   const int32_t* cu; const int32_t* ycu;
   int total_x, total_y, batch, H, ks, st;
   long long xsn, xsh, ysn, ysh, dysn, dysh, dxsn, dxsh;  // w, dw: [H, ks*D, D] contiguous
-  float* partial; int splits;                            // forward split over the contraction: fp32 [splits][total_y][H][D]
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -50,91 +49,127 @@ __device__ __forceinline__ int slot_sequence(const int32_t* __restrict__ cu, int
 }
 
 // ------------------------------------------------------------------------------------------
-template <typename T, int D>
-__global__ __launch_bounds__(256) void lin_fwd_kernel(LinParams p) {
+// Forward.  A workgroup = 16*NT output rows of one head; its 8 waves split the window positions and add their
+// fp32 sums through LDS in a fixed order.  Nothing is staged: per 32 contraction rows (a "chunk") a lane loads
+// an 8 x (D/16) piece of W, rows d = 32q + 8*lg + 0..7, columns e = (D/16)*li + 0..D/16-1 (a wave reads 4 whole rows per
+// load), and transposes it in its own registers with byte permutes into D/16 operand fragments: fragment j holds
+// W[d.., (D/16)*li + j].  MFMA j therefore produces the output columns e = (D/16)*m + j, m the row index of its A
+// operand, and a lane ends up with D/4 consecutive columns of one output row.  All loads of several chunks are in
+// flight at once and there is no barrier before the final sum.
+template <typename T, int D, int NT>
+__global__ __launch_bounds__(512) void lin_fwd_kernel(LinParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NET = D / 16, LD = lds_pitch(D), PIECES = 32 * (D / 8), PPT = (PIECES + 255) / 256;
-  __shared__ __attribute__((aligned(16))) T w_s[2][32][LD];
+  constexpr int NJ = D / 16, NW = D / 32, ROWS = 16 * NT, LP = D + 4;
+  constexpr int GC0 = (NT == 1 ? 16 : NT == 2 ? 12 : 8) / NW, GC = GC0 < 1 ? 1 : GC0 > 8 ? 8 : GC0;   // chunks loaded together: at most 128 registers of W
+  constexpr int VW = NW % 4 == 0 ? 4 : NW % 2 == 0 ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) float part[4][ROWS][LP];
   const int h = blockIdx.y;
-  const int b = slot_sequence(p.ycu, p.batch, blockIdx.x, 64);
+  const int b = slot_sequence(p.ycu, p.batch, blockIdx.x, ROWS);
   const int ylen = p.ycu[b + 1] - p.ycu[b];
-  const int n0 = (blockIdx.x - first_slot_of(p.ycu, b, 64)) * 64;
+  const int n0 = (blockIdx.x - first_slot_of(p.ycu, b, ROWS)) * ROWS;
   if (n0 >= ylen) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
-  const int n = n0 + 16 * wave + li;
-  const bool live = n < ylen;
-  const T* xrow = (const T*)p.x + (long long)(p.cu[b] + (live ? n : 0) * p.st) * p.xsn + (long long)h * p.xsh;
-  const T* wh = (const T*)p.w + (long long)h * p.ks * D * D;
-  f32x4 acc[NET];
+  const T* xrow[NT];
+  bool live[NT];
 #pragma unroll
-  for (int i = 0; i < NET; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // W tile staging registers.  The loads and the LDS writes are written out at their three places of use:
-  // as lambdas over a register array the array ended up in scratch memory.
-  uint4 regs[PPT];
-#define LIN_FETCH(STEP)                                                                                              \
-  _Pragma("unroll") for (int u = 0; u < PPT; u++) {                                                                  \
-    const int pc = min(tid + u * 256, PIECES - 1);                                                                   \
-    regs[u] = *reinterpret_cast<const uint4*>(wh + ((long long)(STEP) * 32 + pc / (D / 8)) * D + (pc % (D / 8)) * 8); \
+  for (int t = 0; t < NT; t++) {
+    const int n = n0 + 16 * t + li;
+    live[t] = n < ylen;
+    xrow[t] = (const T*)p.x + (long long)(p.cu[b] + (live[t] ? n : 0) * p.st) * p.xsn + (long long)h * p.xsh + 8 * lg;
   }
-#define LIN_STASH(BUF)                                                                                               \
-  _Pragma("unroll") for (int u = 0; u < PPT; u++) {                                                                  \
-    const int pc = tid + u * 256;                                                                                    \
-    if (pc < PIECES) *reinterpret_cast<uint4*>(&w_s[BUF][pc / (D / 8)][(pc % (D / 8)) * 8]) = regs[u];               \
+  const T* wl = (const T*)p.w + (long long)h * p.ks * D * D + (long long)(8 * lg) * D + NJ * li;
+  f32x4 acc[NT][NJ];
+#pragma unroll
+  for (int t = 0; t < NT; t++)
+#pragma unroll
+    for (int j = 0; j < NJ; j++) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // this wave's window positions, as chunks of 32 rows of W[h]
+  const int per = (p.ks + 7) / 8;
+  const int q0 = min(p.ks, wave * per) * NW, q1 = min(p.ks, (wave + 1) * per) * NW;
+  for (int g = q0; g < q1; g += GC) {
+    uint32_t wr[GC][8][NW];
+    v8 xf[GC][NT];
+#pragma unroll
+    for (int u = 0; u < GC; u++) {
+      const int q = min(g + u, q1 - 1);   // a short last group loads its last chunk again and does not use it
+      const T* wq = wl + (long long)q * 32 * D;
+#pragma unroll
+      for (int r = 0; r < 8; r++)
+#pragma unroll
+        for (int w0 = 0; w0 < NW; w0 += VW) {
+          if constexpr (VW == 4) {
+            const uint4 t4 = *reinterpret_cast<const uint4*>(wq + r * D + 2 * w0);
+            wr[u][r][w0] = t4.x; wr[u][r][w0 + 1] = t4.y; wr[u][r][w0 + 2] = t4.z; wr[u][r][w0 + 3] = t4.w;
+          } else if constexpr (VW == 2) {
+            const uint2 t2 = *reinterpret_cast<const uint2*>(wq + r * D + 2 * w0);
+            wr[u][r][w0] = t2.x; wr[u][r][w0 + 1] = t2.y;
+          } else {
+            wr[u][r][w0] = *reinterpret_cast<const uint32_t*>(wq + r * D + 2 * w0);
+          }
+        }
+      const int k = q / NW, c = q % NW;
+#pragma unroll
+      for (int t = 0; t < NT; t++) xf[u][t] = live[t] ? ld16<v8>(xrow[t] + (long long)k * p.xsn + 32 * c) : zero16<v8>();
+    }
+#pragma unroll
+    for (int u = 0; u < GC; u++) {
+      if (g + u < q1) {
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+          // 16-bit column j of the lane's 8 x NJ piece: element r comes from row r
+          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+          uint4 f;
+          f.x = __builtin_amdgcn_perm(wr[u][1][j >> 1], wr[u][0][j >> 1], sel);
+          f.y = __builtin_amdgcn_perm(wr[u][3][j >> 1], wr[u][2][j >> 1], sel);
+          f.z = __builtin_amdgcn_perm(wr[u][5][j >> 1], wr[u][4][j >> 1], sel);
+          f.w = __builtin_amdgcn_perm(wr[u][7][j >> 1], wr[u][6][j >> 1], sel);
+          const v8 wf = __builtin_bit_cast(v8, f);
+#pragma unroll
+          for (int t = 0; t < NT; t++) acc[t][j] = E::mfma16(wf, xf[u][t], acc[t][j]);
+        }
+      }
+    }
   }
-  // step = (k, 32-wide slice of d): rows [32*step, +32) of W[h]; blockIdx.z takes a contiguous share of the steps
-  const int all_steps = p.ks * NK, per = (all_steps + p.splits - 1) / p.splits;
-  const int step0 = blockIdx.z * per, n_steps = min(all_steps, step0 + per);
-  if (step0 < n_steps) {
-    LIN_FETCH(step0)
-    LIN_STASH(step0 & 1)
+  // acc[t][j][r] = y[n0 + 16t + li][NJ * (4*lg + r) + j]: the lane's D/4 columns start at D/4 * lg, in (r, j) order.
+  // Waves 4..7 hand their sums to waves 0..3, those hand theirs to all threads: ((w0 + w4) + (w1 + w5)) + ((w2 + w6) + (w3 + w7)).
+  auto stash = [&](int slot) {
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+      for (int i = 0; i < 4 * NJ; i += 4) {
+        f32x4 o;
+#pragma unroll
+        for (int z = 0; z < 4; z++) o[z] = acc[t][(i + z) % NJ][(i + z) / NJ];
+        *reinterpret_cast<f32x4*>(&part[slot][16 * t + li][4 * NJ * lg + i]) = o;
+      }
+  };
+  if (wave >= 4) stash(wave - 4);
+  __syncthreads();
+  if (wave < 4) {
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+      for (int i = 0; i < 4 * NJ; i += 4) {
+        const f32x4 o = *reinterpret_cast<const f32x4*>(&part[wave][16 * t + li][4 * NJ * lg + i]);
+#pragma unroll
+        for (int z = 0; z < 4; z++) acc[t][(i + z) % NJ][(i + z) / NJ] += o[z];
+      }
   }
   __syncthreads();
-  for (int step = step0; step < n_steps; step++) {
-    const int buf = step & 1;
-    const int nxt = min(step + 1, n_steps - 1);   // the last trip loads its own tile again and does not store it
-    LIN_FETCH(nxt)
-    const int k = step / NK, c = step % NK;
-    const v8 xf = row_frag<T>(xrow + (long long)k * p.xsn, 32 * c, lg, live);
+  if (wave < 4) stash(wave);
+  __syncthreads();
+  for (int i = tid; i < ROWS * (D / 4); i += 512) {
+    const int row = i / (D / 4), c4 = 4 * (i % (D / 4));
+    if (n0 + row >= ylen) continue;
+    const f32x4 s = (*reinterpret_cast<const f32x4*>(&part[0][row][c4]) + *reinterpret_cast<const f32x4*>(&part[1][row][c4])) +
+                    (*reinterpret_cast<const f32x4*>(&part[2][row][c4]) + *reinterpret_cast<const f32x4*>(&part[3][row][c4]));
+    v4 o;
 #pragma unroll
-    for (int et = 0; et < NET; et++) acc[et] = E::mfma16(lds_tr_frag<T, LD>(w_s[buf], 16 * et, li, lg), xf, acc[et]);
-    if (step + 1 < n_steps) { LIN_STASH(buf ^ 1) }
-    __syncthreads();
+    for (int z = 0; z < 4; z++) o[z] = (T)s[z];
+    st8((T*)p.y + (long long)(p.ycu[b] + n0 + row) * p.ysn + (long long)h * p.ysh + c4, o);
   }
-#undef LIN_FETCH
-#undef LIN_STASH
-  if (live && p.splits == 1) {
-    T* yp = (T*)p.y + (long long)(p.ycu[b] + n) * p.ysn + (long long)h * p.ysh + 4 * lg;
-#pragma unroll
-    for (int et = 0; et < NET; et++) {
-      v4 o;
-#pragma unroll
-      for (int r = 0; r < 4; r++) o[r] = (T)acc[et][r];
-      st8(yp + 16 * et, o);
-    }
-  } else if (live) {
-    float* pp = p.partial + (((long long)blockIdx.z * p.total_y + p.ycu[b] + n) * p.H + h) * D + 4 * lg;
-#pragma unroll
-    for (int et = 0; et < NET; et++) *reinterpret_cast<f32x4*>(pp + 16 * et) = acc[et];
-  }
-}
-
-// y = sum over the splits of the fp32 partials, in a fixed order
-template <typename T, int D>
-__global__ __launch_bounds__(256) void lin_reduce_kernel(LinParams p) {
-  using v4 = typename Elem<T>::v4;
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // (row, head, 4-wide piece)
-  const long long n_pieces = (long long)p.total_y * p.H * (D / 4);
-  if (i >= n_pieces) return;
-  const int c = (int)(i % (D / 4)), h = (int)((i / (D / 4)) % p.H);
-  const long long row = i / ((long long)(D / 4) * p.H);
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int z = 0; z < p.splits; z++) acc += *reinterpret_cast<const f32x4*>(p.partial + (long long)z * p.total_y * p.H * D + i * 4);
-  v4 o;
-#pragma unroll
-  for (int r = 0; r < 4; r++) o[r] = (T)acc[r];
-  st8((T*)p.y + row * p.ysn + (long long)h * p.ysh + 4 * c, o);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -268,10 +303,23 @@ __global__ __launch_bounds__(256) void lin_dw_kernel(LinParams p) {
 template <typename T, int D>
 static int lin_run(const LinParams& p, int what, hipStream_t s) {
   if (what == 0) {
-    const int64_t slots = p.total_y / 64 + p.batch + 1;
+    // Rows per workgroup: W[h] passes through the workgroup's CU once per workgroup, so more rows mean fewer reads
+    // of W, as long as at least 128 workgroups remain.  Measured, kernel 32 stride 16, 4 heads, d=128, inputs cached:
+    // 1021 output rows 18.9 / 23.5 / 30.3 us at 16 / 32 / 64 rows (from memory, between other kernels: 33.7 / 25.5 / 34.2),
+    // 4093 output rows 61.7 / 47.9 / 37.2 us.
     if (p.total_y > 0) {
-      lin_fwd_kernel<T, D><<<dim3((unsigned)slots, (unsigned)p.H, (unsigned)p.splits), 256, 0, s>>>(p);
-      if (p.splits > 1) lin_reduce_kernel<T, D><<<(unsigned)(((long long)p.total_y * p.H * (D / 4) + 255) / 256), 256, 0, s>>>(p);
+      const auto wgs = [&](int rows) { return (p.total_y / rows + p.batch + 1) * (int64_t)p.H; };
+      if constexpr (D <= 128) {
+        if (wgs(64) >= 128) {
+          lin_fwd_kernel<T, D, 4><<<dim3((unsigned)(wgs(64) / p.H), (unsigned)p.H), 512, 0, s>>>(p);
+          return nsa_check_launch();
+        }
+        if (wgs(32) >= 128) {
+          lin_fwd_kernel<T, D, 2><<<dim3((unsigned)(wgs(32) / p.H), (unsigned)p.H), 512, 0, s>>>(p);
+          return nsa_check_launch();
+        }
+      }
+      lin_fwd_kernel<T, D, 1><<<dim3((unsigned)(wgs(16) / p.H), (unsigned)p.H), 512, 0, s>>>(p);
     }
   } else {
     const int64_t unit = 64 * (int64_t)p.st;
@@ -303,24 +351,12 @@ static int lin_fill(LinParams& p, const void* x, const void* w, const int32_t* c
   p.x = x; p.w = w; p.cu = cu; p.ycu = ycu; p.total_x = (int)total_x; p.total_y = (int)total_y; p.batch = (int)batch; p.H = (int)H;
   p.ks = (int)ks; p.st = (int)st; p.xsn = xsn; p.xsh = xsh;
   p.dy = nullptr; p.y = nullptr; p.dx = nullptr; p.dw = nullptr; p.ysn = p.ysh = p.dysn = p.dysh = p.dxsn = p.dxsh = 0;
-  p.partial = nullptr; p.splits = 1;
   return NSA_OK;
 }
 
-// The forward has 64 output rows x one head per workgroup and kernel_size * D / 32 dependent steps: a few dozen
-// workgroups for a typical input.  The contraction is therefore split over up to 16 workgroups (fp32 partials,
-// summed in a fixed order) until about a thousand workgroups are in flight.
-static int lin_fwd_splits(int64_t total_y, int64_t batch, int64_t H, int64_t ks, int64_t head_dim) {
-  const int64_t wgs = (total_y / 64 + batch + 1) * H, steps = ks * (head_dim / 32);
-  int splits = 1;
-  while (splits < 16 && wgs * splits < 1024 && steps / (splits * 2) >= 4) splits *= 2;
-  return splits;
-}
-
-extern "C" size_t nsa_linear_compress_fwd_workspace_bytes(int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim, int64_t kernel_size) {
-  const int splits = lin_fwd_splits(total_y, batch, num_heads, kernel_size, head_dim);
-  return splits > 1 ? (size_t)splits * total_y * num_heads * head_dim * 4 : 0;
-}
+// The forward keeps its partial sums in LDS: no workspace.  The query stays so that callers written against a
+// library that needed one keep working.
+extern "C" size_t nsa_linear_compress_fwd_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int64_t) { return 0; }
 
 extern "C" int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
                                        int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
@@ -332,12 +368,7 @@ extern "C" int nsa_linear_compress_fwd(const void* x, const void* w, void* y, co
   if (rc != NSA_OK) return rc;
   if (total_y > 0 && (!y || (y_stride_n | y_stride_h) % 4 != 0 || (uintptr_t)y % 8 != 0)) return NSA_ERR_UNSUPPORTED;
   p.y = y; p.ysn = y_stride_n; p.ysh = y_stride_h;
-  p.splits = lin_fwd_splits(total_y, batch, num_heads, kernel_size, head_dim);
-  if (p.splits > 1) {
-    if (!workspace || (uintptr_t)workspace % 16 != 0) return NSA_ERR_BAD_ARG;
-    if (workspace_bytes < nsa_linear_compress_fwd_workspace_bytes(total_y, batch, num_heads, head_dim, kernel_size)) return NSA_ERR_WORKSPACE;
-    p.partial = (float*)workspace;
-  }
+  (void)workspace; (void)workspace_bytes;
   return lin_dispatch(p, 0, head_dim, dtype, (hipStream_t)stream);
 }
 

@@ -82,11 +82,15 @@ def test_pool_asserts(device):
 
 LINEAR_CASES = [
     # lens, H, d, ks, st, dtype
-    ([1024, 7168, 8192], 4, 128, 32, 16, torch.bfloat16),         # pipeline benchmark shape
+    ([1024, 7168, 8192], 4, 128, 32, 16, torch.bfloat16),         # pipeline benchmark shape (32 rows per workgroup)
     ([12, 100, 257, 64], 2, 64, 32, 16, torch.float16),
     ([300, 75], 3, 96, 16, 16, torch.bfloat16),
     ([500], 2, 192, 32, 16, torch.float16),                        # the reference's d=192 smoke shape
     ([900, 130], 1, 32, 64, 32, torch.bfloat16),
+    ([17000, 40], 4, 64, 16, 4, torch.bfloat16),                   # enough outputs for 64 rows per workgroup
+    ([9000, 8200], 4, 96, 16, 4, torch.float16),                   # the same with d=96
+    ([4200, 4100, 31], 8, 128, 16, 4, torch.bfloat16),             # the same with d=128
+    ([4200, 4100, 31], 2, 32, 16, 4, torch.bfloat16),              # 32 rows per workgroup, d=32
 ]
 
 
