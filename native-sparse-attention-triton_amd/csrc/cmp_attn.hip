@@ -688,7 +688,7 @@ __global__ __launch_bounds__(256) void cmp_segments_kernel(const int32_t* __rest
   }
 }
 
-struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, partial, total; int64_t max_blocks, max_items; int chunk; };
+struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, order, partial, total; int64_t max_blocks, max_items; int chunk; };
 static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
   CmpBwdLayout L;
   L.max_blocks = Tk / 64 + B;
@@ -703,6 +703,7 @@ static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq
   L.seg_begin = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.seg_end = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.chunk_off = take((size_t)(Hkv * L.max_blocks + 1) * 4);
+  L.order = take((size_t)L.max_items * 4);
   L.partial = take((size_t)L.max_items * 64 * D * 4 * 2);
   L.total = off;
   return L;
@@ -754,7 +755,10 @@ static int run_cmp(CmpArgs& a) {
     cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
     cmp_segments_kernel<<<1, 256, (size_t)(a.B + 1) * 4, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
     chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off, L.chunk);
+    int32_t* order = (int32_t*)(a.ws + L.order);
+    item_order_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, chunk_off, n_seg, (int)L.max_blocks, L.chunk, (int)(a.Tq / L.chunk + 1), order);
     DkdvParams d;
+    d.order = order;
     d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
     d.cu_blk = cu_blk; d.seg_begin = seg_begin; d.seg_end = seg_end; d.chunk_off = chunk_off; d.queries = nullptr;
     d.partial = (float*)(a.ws + L.partial);
@@ -762,8 +766,8 @@ static int run_cmp(CmpArgs& a) {
     d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st; d.window = a.p.window; d.chunk = L.chunk;
     d.qsn = (int)a.p.qsn; d.qsh = (int)a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = (int)a.p.dsn; d.dsh = (int)a.p.dsh;
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
-    if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
-    else dkdv_kernel<T, D, 64, true, false><<<(unsigned)L.max_items, 64 * dkdv_waves(64), 0, a.stream>>>(d);
+    if (a.p.GT == 1) dkdv_kernel<T, D, 64, true, true><<<(unsigned)L.max_items + 7, 64 * dkdv_waves(64), 0, a.stream>>>(d);
+    else dkdv_kernel<T, D, 64, true, false><<<(unsigned)L.max_items + 7, 64 * dkdv_waves(64), 0, a.stream>>>(d);
     dkdv_reduce_kernel<T, D, 64><<<dim3((unsigned)n_seg, 8), 256, 0, a.stream>>>(d.partial, chunk_off, a.p.cu_k, cu_blk, (int)a.B, (int)L.max_blocks,
                                                                        (T*)a.dk, (T*)a.dv, a.dksn, a.dksh, a.dvsn, a.dvsh);
   }

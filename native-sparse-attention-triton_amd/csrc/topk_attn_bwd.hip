@@ -481,6 +481,7 @@ static int run_bwd(const BwdArgs& a) {
   }
   if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;
+    p.order = nullptr;
     p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.cu = a.cu;
     p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_begin = (const int32_t*)(ws + L.seg_off); p.seg_end = p.seg_begin + 1;
     p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.queries);

@@ -51,7 +51,7 @@ def test_more_host_side_checks():
     assert rc == -1
     # the linear_compress forward sums the shares of its waves in LDS: no workspace
     assert lib.nsa_linear_compress_fwd_workspace_bytes(1021, 3, 4, 128, 32) == 0
-    assert lib.nsa_linear_compress_fwd_workspace_bytes(200000, 1, 8, 128, 32) == 0          # enough workgroups already
+    assert lib.nsa_linear_compress_fwd_workspace_bytes(200000, 1, 8, 128, 32) == 0
     # a cache update with more sequences than the slab holds
     assert lib.nsa_cache_stage_token(fake, fake, fake, fake, 5, 2, 128, 256, 128, 256, 128, 4, 32, 16, None) == -1
     # rope needs row strides that are multiples of 8 elements
