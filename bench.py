@@ -128,7 +128,7 @@ def bench_pipeline(args, dev):
     f_lin = 2 * 2.0 * int(cuk[-1]) * ks * D * D * HKV
     f_cmp = 4.0 * D * HQ * pairs
     f_top = 4.0 * D * bs * (HQ // HKV) * int((idx >= 0).sum())
-    ops = [("linear_compress (K and V: lin_fwd_kernel + lin_reduce_kernel)", t_lin, f_lin),
+    ops = [("linear_compress (K and V: lin_fwd_kernel, two launches)", t_lin, f_lin),
            ("compressed_attention forward (cmp_fwd_kernel)", t_cmp, f_cmp),
            ("block selection (cmp_select_kernel; recomputes the scores: no algorithmic FLOPs of its own)", t_sel, 0.0),
            ("topk_sparse_attention forward (retile_kernel x2 + topk_fwd_kernel)", t_top, f_top)]
