@@ -447,6 +447,9 @@ def bench_probes(args, dev):
     dst = torch.empty_like(src)
     ms = _time_ms(lambda: pl.nsa_probe_copy(src.data_ptr(), dst.data_ptr(), 1 << 30, st), it, 1)
     probes["copy_1GiB"] = {"ms": round(ms, 4), "TBps_read_plus_write": round(2 * (1 << 30) / ms / 1e9, 2)}
+    # the bytes of one pooling forward at N=65536 (33.5 MB in, 2.1 MB out) as a plain copy: what a launch of that size can reach
+    ms = _time_ms(lambda: pl.nsa_probe_copy(src.data_ptr(), dst.data_ptr(), 17 << 20, st), 10 * it, 1)
+    probes["copy_17MiB"] = {"ms": round(ms, 4), "TBps_read_plus_write": round(2 * (17 << 20) / ms / 1e9, 2)}
     del src, dst
     outf = torch.empty(256 * 16 * 256, dtype=torch.float32, device=dev)
     for shape, per_it in ((16, 8 * 16 * 16 * 32 * 2), (32, 4 * 32 * 32 * 16 * 2)):
