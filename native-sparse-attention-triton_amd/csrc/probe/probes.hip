@@ -105,6 +105,51 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, float* __res
   out[(long long)blockIdx.x * 256 + threadIdx.x] = sum;
 }
 
+// Do the matrix pipe and the vector ALU of a SIMD work at the same time?  Per trip a wave issues 8 independent
+// 16x16x32 MFMAs (MODE & 1) and 8 exp2 + 24 fused multiply-adds on 24 independent registers (MODE & 2), in source
+// order MFMA, 4 vector operations (a multiply-add feeding an exp2, two more multiply-adds), MFMA, ...; MODE & 4 puts
+// four more multiply-adds (same issue time) in the place of the exp2
+template <int MODE>
+__global__ __launch_bounds__(256) void probe_coexec_kernel(int iters, float* __restrict__ out) {
+  bf16x8 a, b;
+  for (int i = 0; i < 8; i++) { a[i] = (__bf16)(threadIdx.x * 0.001f + i); b[i] = (__bf16)(1.f - threadIdx.x * 0.002f); }
+  f32x4 c[8];
+  float x[32];
+  for (int j = 0; j < 8; j++) c[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 32; j++) x[j] = 0.001f * (float)(threadIdx.x + j);
+  const float ka = 0.5f + 1e-6f * (float)threadIdx.x, kb = -0.25f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      if (MODE & 1) {
+        if (MODE & 8) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c[j]) : "v"(a), "v"(b));   // accumulator in AGPRs
+        else c[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c[j], 0, 0, 0);
+      }
+      if (MODE & 2) {
+        if (MODE & 4) { x[4 * j] = __builtin_fmaf(x[4 * j], ka, kb); x[4 * j + 3] = __builtin_fmaf(x[4 * j + 3], ka, kb); x[4 * j] = __builtin_fmaf(x[4 * j], kb, ka); x[4 * j + 3] = __builtin_fmaf(x[4 * j + 3], kb, ka); }
+        else x[4 * j] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[4 * j], ka, kb));
+        x[4 * j + 1] = __builtin_fmaf(x[4 * j + 1], ka, kb);
+        x[4 * j + 2] = __builtin_fmaf(x[4 * j + 2], ka, kb);
+      }
+    }
+  }
+  float sum = 0.f;
+  for (int j = 0; j < 8; j++) sum += c[j][0] + c[j][1] + c[j][2] + c[j][3];
+  for (int j = 0; j < 32; j++) sum += x[j];
+  out[(long long)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+extern "C" int nsa_probe_coexec(int mode, int iters, int n_workgroups, float* out, void* stream) {
+  if (mode == 1) probe_coexec_kernel<1><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (mode == 2) probe_coexec_kernel<2><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (mode == 3) probe_coexec_kernel<3><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (mode == 6) probe_coexec_kernel<6><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (mode == 11) probe_coexec_kernel<11><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (mode == 7) probe_coexec_kernel<7><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else return -2;
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
 extern "C" int nsa_probe_copy(const void* src, void* dst, long long bytes, void* stream) {
   probe_copy_kernel<<<16384, 256, 0, (hipStream_t)stream>>>((const uint4*)src, (uint4*)dst, bytes / 16);
   return hipGetLastError() == hipSuccess ? 0 : -4;
