@@ -460,11 +460,14 @@ def bench_probes(args, dev):
                 "ms": round(ms, 4), "PFLOPs": round(n_wg * 4 * iters * per_it / ms / 1e12, 3)}
     # matrix pipe and vector ALU of a SIMD at once: 8 MFMAs and / or 24 multiply-adds + 8 exp2 per trip, two waves per SIMD
     pl.nsa_probe_coexec.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, P, P]
-    for name, mode in (("mfma_only", 1), ("fma_and_exp2_only", 2), ("mfma_with_fma_and_exp2", 3), ("mfma_in_agprs_with_fma_and_exp2", 11),
-                       ("fma_only", 6), ("mfma_with_fma", 7)):
+    for name, mode, n_wg in (("2_waves_per_simd_mfma_only", 1, 512), ("2_waves_per_simd_fma_and_exp2_only", 2, 512),
+                             ("2_waves_per_simd_mfma_with_fma_and_exp2", 3, 512), ("2_waves_per_simd_mfma_in_agprs_with_fma_and_exp2", 11, 512),
+                             ("2_waves_per_simd_fma_only", 6, 512), ("2_waves_per_simd_mfma_with_fma", 7, 512),
+                             ("1_wave_per_simd_mfma_only", 1, 256), ("1_wave_per_simd_fma_and_exp2_only", 2, 256),
+                             ("1_mfma_wave_and_1_fma_and_exp2_wave_per_simd", 19, 512)):
         iters = 20000
-        ms = _time_ms(lambda: pl.nsa_probe_coexec(mode, iters, 512, outf.data_ptr(), st), 3, 1)
-        probes["coexec_2_waves_per_simd_" + name] = {"ms": round(ms, 4), "clk_per_trip_per_simd_at_2.4GHz": round(ms * 1e-3 * 2.4e9 / iters, 1)}
+        ms = _time_ms(lambda: pl.nsa_probe_coexec(mode, iters, n_wg, outf.data_ptr(), st), 3, 1)
+        probes["coexec_" + name] = {"ms": round(ms, 4), "clk_per_trip_per_simd_at_2.4GHz": round(ms * 1e-3 * 2.4e9 / iters, 1)}
     return {
         "metric": "probes behind the top-k attention roofline (N=%d, top-%d): kernel ms per part of topk_idx, memory-system and MFMA ceilings" % (N, topk),
         "value": parts["all_blocks"]["topk_fwd_kernel"], "unit": "ms", "n_gpus": 1, "steps": it, "warmup": 1,

@@ -6,6 +6,7 @@
 //   nsa_probe_gather_rows   : the access pattern of the dK/dV pass - 4 KiB rows at random offsets of a buffer;
 //   nsa_probe_copy          : a plain copy (reference point for the FETCH_SIZE / WRITE_SIZE counters);
 //   nsa_probe_mfma          : back-to-back independent MFMAs on registers (the matrix-core ceiling).
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -109,6 +110,8 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, float* __res
 // 16x16x32 MFMAs (MODE & 1) and 8 exp2 + 24 fused multiply-adds on 24 independent registers (MODE & 2), in source
 // order MFMA, 4 vector operations (a multiply-add feeding an exp2, two more multiply-adds), MFMA, ...; MODE & 4 puts
 // four more multiply-adds (same issue time) in the place of the exp2
+// MODE & 16: the two kinds of work on different waves of a SIMD: workgroups of the first half of the grid issue only the MFMAs,
+// those of the second half only the vector operations (with 512 workgroups each CU gets one of either kind)
 template <int MODE>
 __global__ __launch_bounds__(256) void probe_coexec_kernel(int iters, float* __restrict__ out) {
   bf16x8 a, b;
@@ -118,20 +121,29 @@ __global__ __launch_bounds__(256) void probe_coexec_kernel(int iters, float* __r
   for (int j = 0; j < 8; j++) c[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < 32; j++) x[j] = 0.001f * (float)(threadIdx.x + j);
   const float ka = 0.5f + 1e-6f * (float)threadIdx.x, kb = -0.25f;
-  for (int it = 0; it < iters; it++) {
+  auto trips = [&](auto with_mfma, auto with_valu) {
+    for (int it = 0; it < iters; it++) {
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      if (MODE & 1) {
-        if (MODE & 8) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c[j]) : "v"(a), "v"(b));   // accumulator in AGPRs
-        else c[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c[j], 0, 0, 0);
-      }
-      if (MODE & 2) {
-        if (MODE & 4) { x[4 * j] = __builtin_fmaf(x[4 * j], ka, kb); x[4 * j + 3] = __builtin_fmaf(x[4 * j + 3], ka, kb); x[4 * j] = __builtin_fmaf(x[4 * j], kb, ka); x[4 * j + 3] = __builtin_fmaf(x[4 * j + 3], kb, ka); }
-        else x[4 * j] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[4 * j], ka, kb));
-        x[4 * j + 1] = __builtin_fmaf(x[4 * j + 1], ka, kb);
-        x[4 * j + 2] = __builtin_fmaf(x[4 * j + 2], ka, kb);
+      for (int j = 0; j < 8; j++) {
+        if (decltype(with_mfma)::value) {
+          if (MODE & 8) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c[j]) : "v"(a), "v"(b));   // accumulator in AGPRs
+          else c[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c[j], 0, 0, 0);
+        }
+        if (decltype(with_valu)::value) {
+          if (MODE & 4) { x[4 * j] = __builtin_fmaf(x[4 * j], ka, kb); x[4 * j + 3] = __builtin_fmaf(x[4 * j + 3], ka, kb); x[4 * j] = __builtin_fmaf(x[4 * j], kb, ka); x[4 * j + 3] = __builtin_fmaf(x[4 * j + 3], kb, ka); }
+          else x[4 * j] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[4 * j], ka, kb));
+          x[4 * j + 1] = __builtin_fmaf(x[4 * j + 1], ka, kb);
+          x[4 * j + 2] = __builtin_fmaf(x[4 * j + 2], ka, kb);
+        }
       }
     }
+  };
+  using yes = std::true_type;
+  using no = std::false_type;
+  if (MODE & 16) {
+    if (blockIdx.x < gridDim.x / 2) trips(yes{}, no{}); else trips(no{}, yes{});
+  } else {
+    trips(std::integral_constant<bool, (MODE & 1) != 0>{}, std::integral_constant<bool, (MODE & 2) != 0>{});
   }
   float sum = 0.f;
   for (int j = 0; j < 8; j++) sum += c[j][0] + c[j][1] + c[j][2] + c[j][3];
@@ -145,6 +157,7 @@ extern "C" int nsa_probe_coexec(int mode, int iters, int n_workgroups, float* ou
   else if (mode == 3) probe_coexec_kernel<3><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
   else if (mode == 6) probe_coexec_kernel<6><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
   else if (mode == 11) probe_coexec_kernel<11><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
+  else if (mode == 19) probe_coexec_kernel<19><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
   else if (mode == 7) probe_coexec_kernel<7><<<n_workgroups, 256, 0, (hipStream_t)stream>>>(iters, out);
   else return -2;
   return hipGetLastError() == hipSuccess ? 0 : -4;
