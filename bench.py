@@ -131,7 +131,7 @@ def bench_pipeline(args, dev):
     ops = [("linear_compress (K and V: lin_fwd_kernel, two launches)", t_lin, f_lin),
            ("compressed_attention forward (cmp_fwd_kernel)", t_cmp, f_cmp),
            ("block selection (cmp_select_kernel; recomputes the scores: no algorithmic FLOPs of its own)", t_sel, 0.0),
-           ("topk_sparse_attention forward (retile_kernel x2 + topk_fwd_kernel)", t_top, f_top)]
+           ("topk_sparse_attention forward (retile_pair_kernel + topk_fwd_kernel)", t_top, f_top)]
     roof = _mfma_roofline(ops, (f_lin + f_cmp + f_top) / t_all / 1e9)
     return {
         "roofline": roof,

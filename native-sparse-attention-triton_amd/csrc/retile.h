@@ -26,9 +26,8 @@ enum { RETILE_ROWS = 0, RETILE_COLS = 1 };
 __device__ __forceinline__ int seq_first_slot(const int32_t* __restrict__ cu, int b) { return (cu[b] + 31) / 32 + b; }
 
 template <typename T, int D, int MODE>
-__global__ __launch_bounds__(256) void retile_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu, int batch,
-                                                     long long stride_n, long long stride_h, int n_slots) {
-  __shared__ __attribute__((aligned(16))) T tile[32][lds_pitch(D)];
+__device__ __forceinline__ void retile_body(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu, int batch,
+                                            long long stride_n, long long stride_h, int n_slots, T (*tile)[lds_pitch(D)]) {
   const int slot = blockIdx.x, h = blockIdx.y;
   int lo = 0, hi = batch;
   while (hi - lo > 1) {
@@ -67,10 +66,34 @@ __global__ __launch_bounds__(256) void retile_kernel(const T* __restrict__ x, T*
 }
 
 template <typename T, int D, int MODE>
+__global__ __launch_bounds__(256) void retile_kernel(const T* __restrict__ x, T* __restrict__ out, const int32_t* __restrict__ cu, int batch,
+                                                     long long stride_n, long long stride_h, int n_slots) {
+  __shared__ __attribute__((aligned(16))) T tile[32][lds_pitch(D)];
+  retile_body<T, D, MODE>(x, out, cu, batch, stride_n, stride_h, n_slots, tile);
+}
+
+// two tensors of the same shape (K and V) in one launch: blockIdx.z picks the tensor and its layout
+template <typename T, int D, int MODE0, int MODE1>
+__global__ __launch_bounds__(256) void retile_pair_kernel(const T* __restrict__ x0, T* __restrict__ out0, long long sn0, long long sh0,
+                                                          const T* __restrict__ x1, T* __restrict__ out1, long long sn1, long long sh1,
+                                                          const int32_t* __restrict__ cu, int batch, int n_slots) {
+  __shared__ __attribute__((aligned(16))) T tile[32][lds_pitch(D)];
+  if (blockIdx.z == 0) retile_body<T, D, MODE0>(x0, out0, cu, batch, sn0, sh0, n_slots, tile);
+  else retile_body<T, D, MODE1>(x1, out1, cu, batch, sn1, sh1, n_slots, tile);
+}
+
+template <typename T, int D, int MODE>
 static inline void launch_retile(const T* x, T* out, const int32_t* cu, int64_t batch, int64_t stride_n, int64_t stride_h,
                                  int64_t n_slots, int64_t heads, hipStream_t stream) {
   dim3 grid((unsigned)n_slots, (unsigned)heads);
   retile_kernel<T, D, MODE><<<grid, 256, 0, stream>>>(x, out, cu, (int)batch, stride_n, stride_h, (int)n_slots);
+}
+
+template <typename T, int D, int MODE0, int MODE1>
+static inline void launch_retile_pair(const T* x0, T* out0, int64_t sn0, int64_t sh0, const T* x1, T* out1, int64_t sn1, int64_t sh1,
+                                      const int32_t* cu, int64_t batch, int64_t n_slots, int64_t heads, hipStream_t stream) {
+  dim3 grid((unsigned)n_slots, (unsigned)heads, 2);
+  retile_pair_kernel<T, D, MODE0, MODE1><<<grid, 256, 0, stream>>>(x0, out0, sn0, sh0, x1, out1, sn1, sh1, cu, (int)batch, (int)n_slots);
 }
 
 // bytes of one fragment-major copy

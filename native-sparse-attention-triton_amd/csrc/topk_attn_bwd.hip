@@ -466,8 +466,7 @@ static int run_bwd(const BwdArgs& a) {
     DqParams p;
     T* kf = (T*)(ws + L.kf);
     T* vf = (T*)(ws + L.vf);
-    launch_retile<T, D, RETILE_ROWS>((const T*)a.k, kf, a.cu, a.B, a.ksn, a.ksh, L.n_slots, a.Hkv, a.stream);
-    launch_retile<T, D, RETILE_ROWS>((const T*)a.v, vf, a.cu, a.B, a.vsn, a.vsh, L.n_slots, a.Hkv, a.stream);
+    launch_retile_pair<T, D, RETILE_ROWS, RETILE_ROWS>((const T*)a.k, kf, a.ksn, a.ksh, (const T*)a.v, vf, a.vsn, a.vsh, a.cu, a.B, L.n_slots, a.Hkv, a.stream);
     p.q = a.q; p.kf = kf; p.vf = vf; p.dout = a.dout; p.lse = a.lse; p.o = fused_delta ? a.o : nullptr; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk; p.n_slots = (int)L.n_slots;
     p.n_items = (long long)a.T * GT * a.Hkv;

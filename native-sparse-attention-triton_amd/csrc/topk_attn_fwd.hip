@@ -182,8 +182,7 @@ template <typename T, int D, int BS>
 static int launch_fwd(const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn, long long vsh,
                       int phases, hipStream_t stream) {
   if (phases & NSA_FWD_PHASE_TRANSPOSE) {
-    launch_retile<T, D, RETILE_ROWS>((const T*)k, (T*)p.kf, p.cu, p.batch, ksn, ksh, p.n_slots, p.Hkv, stream);
-    launch_retile<T, D, RETILE_COLS>((const T*)v, (T*)p.vf, p.cu, p.batch, vsn, vsh, p.n_slots, p.Hkv, stream);
+    launch_retile_pair<T, D, RETILE_ROWS, RETILE_COLS>((const T*)k, (T*)p.kf, ksn, ksh, (const T*)v, (T*)p.vf, vsn, vsh, p.cu, p.batch, p.n_slots, p.Hkv, stream);
   }
   if (phases & NSA_FWD_PHASE_ATTEND) {
     long long n_wg = (p.n_items + 3) / 4;
