@@ -21,12 +21,16 @@ static constexpr int MAX_CHUNK_TOKENS = 960;
 
 // Queries per work item, from the number of (query, key block) pairs of the launch: long items amortise the
 // loading of K/V and the partial they write, but a launch needs a few thousand items to fill 256 CUs three
-// workgroups deep and to even out the one segment every token selects (its chunks are the longest items).
-// `longest` is the size used by big launches (measured best: 768 for query lists, 960 for query ranges).
+// workgroups deep and to even out the one segment every token selects (its chunks are the longest items); a small
+// launch lasts as long as its longest item (two queries per step, about 1.3 us a step).
+// `longest` is the size used by big launches (measured best: 768 for query lists, 960 for query ranges); the
+// smaller sizes are the measured best of 64..768 at 2048..16384 tokens with 8 and 16 blocks per token
+// (2048 tokens, 8 blocks: backward 0.30 -> 0.26 ms against one size of 256 below 256 Ki pairs).
 static inline int dkdv_chunk_tokens(long long pairs, int longest) {
   if (pairs >= 2048ll * 1024) return longest < MAX_CHUNK_TOKENS ? longest : MAX_CHUNK_TOKENS;
   if (pairs >= 256ll * 1024) return 384;
-  return 256;
+  if (pairs >= 96ll * 1024) return 192;
+  return 128;
 }
 
 // Waves per dK/dV workgroup; each wave owns bs / (16 * waves) key tiles.  Every wave reads all staged
