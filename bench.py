@@ -405,6 +405,35 @@ def bench_probes(args, dev):
         "dkdv_kernel": None}
     del q2, do2, k2, v2, o2, lse2, g2, ws_f2, ws_b2, idx2
 
+    # The same with contiguous key ranges of equal work: R copies of every kv-head, copy r keeps the selected blocks of range r
+    # (a fraction x of the keys holds x (1 + ln 1/x) of the pairs of a causal, uniformly random selection); forward only.
+    import math
+
+    def key_fraction(f):
+        lo, hi = 1e-9, 1.0
+        for _ in range(60):
+            mid = (lo + hi) / 2
+            lo, hi = (mid, hi) if mid * (1 + math.log(1 / mid)) < f else (lo, mid)
+        return lo
+    nb = (N + BS - 1) // BS
+    for R in (2, 4, 8):
+        bounds = [0] + [max(1, round(nb * key_fraction(i / R))) for i in range(1, R)] + [nb]
+        ixs = []
+        for h in range(HKV):
+            for r in range(R):
+                x = torch.where((idx[h] >= bounds[r]) & (idx[h] < bounds[r + 1]), idx[h], torch.full_like(idx[h], 1 << 30)).sort(-1).values
+                ixs.append(torch.where(x == (1 << 30), torch.full_like(x, -1), x))
+        idx_r = torch.stack(ixs, 0).contiguous()
+        k_r, v_r = k.repeat_interleave(R, 1).contiguous(), v.repeat_interleave(R, 1).contiguous()
+        q_r = q.view(N, HKV, 1, HQ // HKV, D).expand(N, HKV, R, HQ // HKV, D).reshape(N, R * HQ, D).contiguous()
+        ws_r = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, R * HKV, D), dev)
+        o_r, lse_r = _topk_sparse_attention_fwd(q_r, k_r, v_r, idx_r, BS, cu, cu, N, N, sm, workspace=ws_r)
+        parts["key_range_split_%d_ranges_of_equal_work_emulated" % R] = {
+            "pairs": int((idx_r >= 0).sum()),
+            "topk_fwd_kernel": round(_time_ms(lambda: _topk_sparse_attention_fwd(q_r, k_r, v_r, idx_r, BS, cu, cu, N, N, sm, workspace=ws_r, phases=2, out=(o_r, lse_r)), it, 1), 4),
+            "dq_kernel": None, "dkdv_kernel": None}
+        del idx_r, k_r, v_r, q_r, ws_r, o_r, lse_r
+
     pl = ctypes.CDLL(os.path.join(os.path.dirname(_lib.lib_path()), "libnsa_probe.so"))
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P, LL, I = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
