@@ -332,181 +332,6 @@ def bench_layer(args, dev):
     }
 
 
-def bench_probes(args, dev):
-    """Evidence behind the roofline discussion of the top-k kernels at the headline shape (N=32768, top-16), one JSON line:
-    which part of topk_idx costs what (forced blocks removed / forced blocks only / one quarter of the sequence at a
-    time), and the rates the memory system and the matrix cores deliver for the kernels' access patterns
-    (libnsa_probe.so: block gather without arithmetic, random 4 KiB rows, plain copy, back-to-back MFMAs)."""
-    import ctypes
-
-    from native_sparse_attention import _lib
-    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
-    from native_sparse_attention.testing import cu_from_lens, make_topk_idx
-
-    N, topk = args.seqlen, args.topk
-    g = torch.Generator(device=dev).manual_seed(0)
-    cu = cu_from_lens([N], dev)
-    q = torch.randn(N, HQ, D, generator=g, device=dev).bfloat16()
-    k = torch.randn(N, HKV, D, generator=g, device=dev).bfloat16()
-    v = torch.randn(N, HKV, D, generator=g, device=dev).bfloat16()
-    do = torch.randn(N, HQ, D, generator=g, device=dev).bfloat16()
-    idx = make_topk_idx(cu, BS, topk, HKV, seed=0, local_blocks=2)
-    sm = D ** -0.5
-    lib = _lib.load()
-    ws_f = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, HKV, D), dev)
-    ws_b = _lib.workspace(lib.nsa_topk_attn_bwd_workspace_bytes(N, 1, HQ, HKV, D, topk, BS), dev)
-    it = max(3, min(args.steps, 10))
-
-    def kernels_ms(ix):
-        o, lse = _topk_sparse_attention_fwd(q, k, v, ix, BS, cu, cu, N, N, sm, workspace=ws_f)
-        grads = _topk_sparse_attention_bwd(o, do, lse, q, k, v, ix, BS, cu, cu, N, N, sm, workspace=ws_b)
-        f = _time_ms(lambda: _topk_sparse_attention_fwd(q, k, v, ix, BS, cu, cu, N, N, sm, workspace=ws_f, phases=2, out=(o, lse)), it, 1)
-        dq = _time_ms(lambda: _topk_sparse_attention_bwd(o, do, lse, q, k, v, ix, BS, cu, cu, N, N, sm, workspace=ws_b, phases=4, out=grads), it, 1)
-        _topk_sparse_attention_bwd(o, do, lse, q, k, v, ix, BS, cu, cu, N, N, sm, workspace=ws_b, phases=1, out=grads)   # index of this ix
-        dkdv = _time_ms(lambda: _topk_sparse_attention_bwd(o, do, lse, q, k, v, ix, BS, cu, cu, N, N, sm, workspace=ws_b, phases=2, out=grads), it, 1)
-        return {"pairs": int((ix >= 0).sum()), "topk_fwd_kernel": round(f, 4), "dq_kernel": round(dq, 4), "dkdv_kernel": round(dkdv, 4)}
-
-    qb = (torch.arange(N, device=dev) // BS)[None, :, None]
-    forced = (idx == 0) | (idx == qb) | (idx == qb - 1)
-
-    def keep(mask):
-        x = torch.where(mask & (idx >= 0), idx, torch.full_like(idx, 1 << 30)).sort(-1).values
-        return torch.where(x == (1 << 30), torch.full_like(x, -1), x).contiguous()
-
-    def rows(lo, hi):
-        ix = torch.full_like(idx, -1)
-        ix[:, lo:hi] = idx[:, lo:hi]
-        return ix
-
-    parts = {"all_blocks": kernels_ms(idx), "forced_blocks_removed": kernels_ms(keep(~forced)), "forced_blocks_only": kernels_ms(keep(forced))}
-    for j in range(4):
-        parts["tokens_quarter_%d_only" % j] = kernels_ms(rows(j * N // 4, (j + 1) * N // 4))
-    parts["tokens_first_half_only"] = kernels_ms(rows(0, N // 2))
-    parts["tokens_second_half_only"] = kernels_ms(rows(N // 2, N))
-
-    # Emulation of a key-range split over the XCDs of a head: kv-head 2h + p = kv-head h restricted to the selected blocks of
-    # parity p (q, k, v duplicated), so that every XCD owns one (head, parity) stream of all tokens and its L2 caches half the blocks.
-    # What a split forward / dQ pass would take before it merged its partial outputs.
-    def parity(pp):
-        x = torch.where((idx >= 0) & (idx % 2 == pp), idx, torch.full_like(idx, 1 << 30)).sort(-1).values
-        return torch.where(x == (1 << 30), torch.full_like(x, -1), x)
-    idx2 = torch.stack([parity(0), parity(1)], 1).reshape(2 * HKV, N, topk).contiguous()
-    k2, v2 = k.repeat_interleave(2, 1).contiguous(), v.repeat_interleave(2, 1).contiguous()
-    q2 = q.view(N, HKV, 1, HQ // HKV, D).expand(N, HKV, 2, HQ // HKV, D).reshape(N, 2 * HQ, D).contiguous()
-    do2 = do.view(N, HKV, 1, HQ // HKV, D).expand(N, HKV, 2, HQ // HKV, D).reshape(N, 2 * HQ, D).contiguous()
-    ws_f2 = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, 2 * HKV, D), dev)
-    ws_b2 = _lib.workspace(lib.nsa_topk_attn_bwd_workspace_bytes(N, 1, 2 * HQ, 2 * HKV, D, topk, BS), dev)
-    o2, lse2 = _topk_sparse_attention_fwd(q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_f2)
-    g2 = _topk_sparse_attention_bwd(o2, do2, lse2, q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_b2)
-    parts["block_parity_split_over_the_two_xcds_of_a_head_emulated"] = {
-        "pairs": int((idx2 >= 0).sum()),
-        "topk_fwd_kernel": round(_time_ms(lambda: _topk_sparse_attention_fwd(q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_f2, phases=2, out=(o2, lse2)), it, 1), 4),
-        "dq_kernel": round(_time_ms(lambda: _topk_sparse_attention_bwd(o2, do2, lse2, q2, k2, v2, idx2, BS, cu, cu, N, N, sm, workspace=ws_b2, phases=4, out=g2), it, 1), 4),
-        "dkdv_kernel": None}
-    del q2, do2, k2, v2, o2, lse2, g2, ws_f2, ws_b2, idx2
-
-    # The same with contiguous key ranges of equal work: R copies of every kv-head, copy r keeps the selected blocks of range r
-    # (a fraction x of the keys holds x (1 + ln 1/x) of the pairs of a causal, uniformly random selection); forward only.
-    import math
-
-    def key_fraction(f):
-        lo, hi = 1e-9, 1.0
-        for _ in range(60):
-            mid = (lo + hi) / 2
-            lo, hi = (mid, hi) if mid * (1 + math.log(1 / mid)) < f else (lo, mid)
-        return lo
-    nb = (N + BS - 1) // BS
-    for R in (2, 4, 8):
-        bounds = [0] + [max(1, round(nb * key_fraction(i / R))) for i in range(1, R)] + [nb]
-        ixs = []
-        for h in range(HKV):
-            for r in range(R):
-                x = torch.where((idx[h] >= bounds[r]) & (idx[h] < bounds[r + 1]), idx[h], torch.full_like(idx[h], 1 << 30)).sort(-1).values
-                ixs.append(torch.where(x == (1 << 30), torch.full_like(x, -1), x))
-        idx_r = torch.stack(ixs, 0).contiguous()
-        k_r, v_r = k.repeat_interleave(R, 1).contiguous(), v.repeat_interleave(R, 1).contiguous()
-        q_r = q.view(N, HKV, 1, HQ // HKV, D).expand(N, HKV, R, HQ // HKV, D).reshape(N, R * HQ, D).contiguous()
-        ws_r = _lib.workspace(lib.nsa_topk_attn_fwd_workspace_bytes(N, 1, R * HKV, D), dev)
-        o_r, lse_r = _topk_sparse_attention_fwd(q_r, k_r, v_r, idx_r, BS, cu, cu, N, N, sm, workspace=ws_r)
-        parts["key_range_split_%d_ranges_of_equal_work_emulated" % R] = {
-            "pairs": int((idx_r >= 0).sum()),
-            "topk_fwd_kernel": round(_time_ms(lambda: _topk_sparse_attention_fwd(q_r, k_r, v_r, idx_r, BS, cu, cu, N, N, sm, workspace=ws_r, phases=2, out=(o_r, lse_r)), it, 1), 4),
-            "dq_kernel": None, "dkdv_kernel": None}
-        del idx_r, k_r, v_r, q_r, ws_r, o_r, lse_r
-
-    pl = ctypes.CDLL(os.path.join(os.path.dirname(_lib.lib_path()), "libnsa_probe.so"))
-    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    P, LL, I = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
-    pl.nsa_probe_copy.argtypes = [P, P, LL, P]
-    pl.nsa_probe_gather_blocks.argtypes = [P, P, P, I, I, I, I, I, P, P]
-    pl.nsa_probe_gather_rows.argtypes = [P, LL, I, I, I, P, P]
-    pl.nsa_probe_tile_gather.argtypes = [P, P, P, I, I, I, I, P, P, P]
-    pl.nsa_probe_mfma.argtypes = [I, I, I, P, P]
-    # block gather on the K / V fragment copies the forward left in its workspace
-    _topk_sparse_attention_fwd(q, k, v, idx, BS, cu, cu, N, N, sm, workspace=ws_f)
-    n_slots = (N + 31) // 32 + 2
-    copy_bytes = HKV * n_slots * 32 * D * 2
-    sink = torch.empty(N * HKV * 64 * 16, dtype=torch.uint8, device=dev)
-    idx_c = idx.contiguous()
-    n_blocks = int((idx >= 0).sum())
-
-    def gather(fold):
-        assert pl.nsa_probe_gather_blocks(ws_f.data_ptr(), ws_f.data_ptr() + copy_bytes, idx_c.data_ptr(), N, HKV, topk, n_slots, fold,
-                                          sink.data_ptr(), st) == 0
-    probes = {}
-    for name, fold in (("gather_blocks_real_ids", 0), ("gather_blocks_folded_into_2MiB_per_head", 64)):
-        ms = _time_ms(lambda: gather(fold), it, 1)
-        probes[name] = {"ms": round(ms, 4), "TBps_into_the_CUs": round(n_blocks * 32768 / ms / 1e9, 2)}
-    if topk <= 32 and N <= 131072:
-        flag = torch.zeros(1, dtype=torch.int32, device=dev)
-        tile = lambda: pl.nsa_probe_tile_gather(ws_f.data_ptr(), ws_f.data_ptr() + copy_bytes, idx_c.data_ptr(), N, HKV, topk, n_slots,
-                                                sink.data_ptr(), flag.data_ptr(), st)
-        ms = _time_ms(tile, it, 1)
-        probes["gather_blocks_shared_in_24_token_tiles_through_LDS_ring"] = {"ms": round(ms, 4), "gave_up": int(flag.item())}
-    # random 4 KiB rows: what the dK/dV pass asks of the memory system
-    for name, mib in (("gather_rows_4KiB_in_1GiB", 1024), ("gather_rows_4KiB_in_128MiB", 128)):
-        buf = torch.empty(mib << 20, dtype=torch.uint8, device=dev).random_()
-        n_wg, reads = 256 * 8 * 2, 512
-        out = torch.empty(n_wg * 4 * 64 * 16, dtype=torch.uint8, device=dev)
-        run = lambda: pl.nsa_probe_gather_rows(buf.data_ptr(), (mib << 20) // 4096, 4096, reads, n_wg, out.data_ptr(), st)
-        ms = _time_ms(run, it, 1)
-        probes[name] = {"ms": round(ms, 4), "TBps": round(n_wg * 4 * reads * 4096 / ms / 1e9, 2)}
-        del buf
-    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()
-    dst = torch.empty_like(src)
-    ms = _time_ms(lambda: pl.nsa_probe_copy(src.data_ptr(), dst.data_ptr(), 1 << 30, st), it, 1)
-    probes["copy_1GiB"] = {"ms": round(ms, 4), "TBps_read_plus_write": round(2 * (1 << 30) / ms / 1e9, 2)}
-    # the bytes of one pooling forward at N=65536 (33.5 MB in, 2.1 MB out) as a plain copy: what a launch of that size can reach
-    ms = _time_ms(lambda: pl.nsa_probe_copy(src.data_ptr(), dst.data_ptr(), 17 << 20, st), 10 * it, 1)
-    probes["copy_17MiB"] = {"ms": round(ms, 4), "TBps_read_plus_write": round(2 * (17 << 20) / ms / 1e9, 2)}
-    del src, dst
-    outf = torch.empty(256 * 16 * 256, dtype=torch.float32, device=dev)
-    for shape, per_it in ((16, 8 * 16 * 16 * 32 * 2), (32, 4 * 32 * 32 * 16 * 2)):
-        for wps in (1, 2, 4):
-            n_wg, iters = 256 * wps, 20000
-            ms = _time_ms(lambda: pl.nsa_probe_mfma(shape, iters, n_wg, outf.data_ptr(), st), 3, 1)
-            probes["mfma_bf16_%dx%d_%d_waves_per_simd" % (shape, shape, wps)] = {
-                "ms": round(ms, 4), "PFLOPs": round(n_wg * 4 * iters * per_it / ms / 1e12, 3)}
-    # matrix pipe and vector ALU of a SIMD at once: 8 MFMAs and / or 24 multiply-adds + 8 exp2 per trip, two waves per SIMD
-    pl.nsa_probe_coexec.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, P, P]
-    for name, mode, n_wg in (("2_waves_per_simd_mfma_only", 1, 512), ("2_waves_per_simd_fma_and_exp2_only", 2, 512),
-                             ("2_waves_per_simd_mfma_with_fma_and_exp2", 3, 512), ("2_waves_per_simd_mfma_in_agprs_with_fma_and_exp2", 11, 512),
-                             ("2_waves_per_simd_fma_only", 6, 512), ("2_waves_per_simd_mfma_with_fma", 7, 512),
-                             ("1_wave_per_simd_mfma_only", 1, 256), ("1_wave_per_simd_fma_and_exp2_only", 2, 256),
-                             ("1_mfma_wave_and_1_fma_and_exp2_wave_per_simd", 19, 512)):
-        iters = 20000
-        ms = _time_ms(lambda: pl.nsa_probe_coexec(mode, iters, n_wg, outf.data_ptr(), st), 3, 1)
-        probes["coexec_" + name] = {"ms": round(ms, 4), "clk_per_trip_per_simd_at_2.4GHz": round(ms * 1e-3 * 2.4e9 / iters, 1)}
-    return {
-        "metric": "probes behind the top-k attention roofline (N=%d, top-%d): kernel ms per part of topk_idx, memory-system and MFMA ceilings" % (N, topk),
-        "value": parts["all_blocks"]["topk_fwd_kernel"], "unit": "ms", "n_gpus": 1, "steps": it, "warmup": 1,
-        "ms_per_step": parts["all_blocks"]["topk_fwd_kernel"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "single sequence N=%d, 64 q / 4 kv heads, d=128, block 64, top-%d" % (N, topk),
-                   "kernel_ms_by_part_of_topk_idx": parts, "probes": probes},
-    }
-
-
 def measure_topk(N, topk, steps, warmup, dev, per_kernel):
     """One point of the top-k sweep: forward + backward of topk_sparse_attention on a single sequence of N tokens (64 q / 4 kv
     heads, d=128, block 64), inputs resident in HBM.  ms_per_step: wall clock over `steps` steps after `warmup`; fwd_ms /
@@ -576,7 +401,7 @@ def main():
                     help="also run three plain 1 GiB device copies (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--readme-heads", action="store_true",
                     help="compressed workload with the 64q/4kv head layout of the reference README tables instead of config 3's 32q/2kv")
-    ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode", "layer", "probes"],
+    ap.add_argument("--workload", default="topk", choices=["topk", "pipeline", "compressed", "decode", "layer"],
                     help="topk = the headline metric (default); the others time the pipeline, long-sequence compressed-attention, decode and whole-layer benchmarks")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -588,7 +413,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload != "topk":
-        fn = {"pipeline": bench_pipeline, "compressed": bench_compressed, "decode": bench_decode, "layer": bench_layer, "probes": bench_probes}[args.workload]
+        fn = {"pipeline": bench_pipeline, "compressed": bench_compressed, "decode": bench_decode, "layer": bench_layer}[args.workload]
         print(json.dumps(fn(args, dev)))
         return
     N, topk = args.seqlen, args.topk

@@ -1,6 +1,5 @@
 """Builds libnsa_hip.so: every csrc/*.hip is compiled for gfx950 with hipcc and linked into one
-C-ABI shared library next to the Python package (native_sparse_attention/lib/).  csrc/probe/*.hip (memory-system
-and MFMA probes that only the benchmark's report uses) go into a library of their own, libnsa_probe.so.
+C-ABI shared library next to the Python package (native_sparse_attention/lib/).
 
     python build.py            # incremental (rebuilds objects older than their sources)
     python build.py --force    # rebuild everything
@@ -16,7 +15,6 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "native_sparse_attention", "lib")
 LIB = os.path.join(LIB_DIR, "libnsa_hip.so")
-PROBE_LIB = os.path.join(LIB_DIR, "libnsa_probe.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wno-unused-value",
@@ -34,7 +32,7 @@ def _newest_header():
 
 
 def _compile(src, force):
-    obj = os.path.join(OBJ, ("probe_" if os.path.dirname(src).endswith("probe") else "") + os.path.basename(src)[:-4] + ".o")
+    obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
     if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _newest_header()):
         return obj
     r = subprocess.run([HIPCC, *FLAGS, "-c", src, "-o", obj], capture_output=True, text=True)
@@ -47,13 +45,11 @@ def build(force=False, jobs=8):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
-    probes = sorted(glob.glob(os.path.join(CSRC, "probe", "*.hip")))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force), srcs + probes))
-    for lib, members in ((LIB, objs[:len(srcs)]), (PROBE_LIB, objs[len(srcs):])):
-        r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members], capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("link failed:\n" + r.stderr[-4000:])
+        objs = list(ex.map(lambda s: _compile(s, force), srcs))
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr[-4000:])
     return LIB
 
 
