@@ -40,13 +40,20 @@ int nsa_version(void);
  * (native_sparse_attention/ops/triton/topk_sparse_attention.py:828-909).
  *   q,o [T,Hq,D]; k,v [T,Hkv,D]; topk_idx int32 [Hkv,T,topk] (entries <0 or beyond the
  *   query's own block are skipped); lse fp32 [Hq,T] in base-2 units (contiguous).
- * workspace holds fragment-major copies of K and V (2x their size): nsa_topk_attn_fwd_workspace_bytes().
+ * workspace holds fragment-major copies of K and V (2x their size) and a 16 KiB pacing table:
+ * nsa_topk_attn_fwd_workspace_bytes().
  * phases: NSA_FWD_PHASE_ALL, or a subset when the caller re-uses the workspace of a previous
  * call with the same K and V (profiling a single kernel).
+ * Schedule: when the K/V rows of one kv-head reach 12 MiB (24 K tokens of 128 columns) the attend pass runs
+ * as persistent waves whose key positions are kept within a window of each other, so that an XCD's L2 serves
+ * most of the block fetches; below that, one wave per token in launch order.  Both give bit-identical
+ * results.  Or-ing NSA_FWD_SCHEDULE_PLAIN or NSA_FWD_SCHEDULE_PACED into phases forces one of them.
  */
 #define NSA_FWD_PHASE_TRANSPOSE 1
 #define NSA_FWD_PHASE_ATTEND 2
 #define NSA_FWD_PHASE_ALL 3
+#define NSA_FWD_SCHEDULE_PLAIN 8
+#define NSA_FWD_SCHEDULE_PACED 16
 size_t nsa_topk_attn_fwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t head_dim);
 int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t* topk_idx, void* o, float* lse,
                       const int32_t* cu_seqlens, int64_t total_len, int64_t batch, int64_t num_q_heads,
@@ -75,11 +82,15 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
  * When PREP and DQ run in the same call, delta = rowsum(o * dout) is formed inside the dQ pass
  * (which runs before dK/dV) instead of by a pass of its own; the stored values are the same.
  * Token strides of q and dout, and group_size * their head strides + D, must fit 31 bits.
+ * The dQ pass has the two schedules of the forward (same rule, same bit-identical results);
+ * NSA_BWD_SCHEDULE_PLAIN / NSA_BWD_SCHEDULE_PACED or-ed into phases force one of them.
  */
 #define NSA_BWD_PHASE_PREP 1
 #define NSA_BWD_PHASE_DKDV 2
 #define NSA_BWD_PHASE_DQ 4
 #define NSA_BWD_PHASE_ALL 7
+#define NSA_BWD_SCHEDULE_PLAIN 8
+#define NSA_BWD_SCHEDULE_PACED 16
 size_t nsa_topk_attn_bwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_q_heads, int64_t num_kv_heads,
                                          int64_t head_dim, int64_t topk, int64_t block_size);
 int64_t nsa_topk_reverse_index_segments(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t block_size);

@@ -17,13 +17,14 @@
 #include <cstring>
 
 #include "retile.h"
+#include "pace.h"
 #include "delta.h"
 #include "dkdv.h"
 
 // ------------------------------------------------------------------------------------------
 // workspace carving (host and entry point must agree)
 struct BwdLayout {
-  size_t delta, cu_blk, hist, queries, seg_off, chunk_off, kf, vf, partial, total;
+  size_t delta, cu_blk, hist, queries, seg_off, chunk_off, kf, vf, pace, partial, total;
   int64_t max_blocks, n_pairs, max_items, n_slots;
   int tile_tokens, n_tiles;
 };
@@ -61,6 +62,7 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   L.n_slots = nsa_chunk_slots(T, B);
   L.kf = take(retile_bytes(T, B, Hkv, D));   // row-fragment copies of K and V for the dQ pass
   L.vf = take(retile_bytes(T, B, Hkv, D));
+  L.pace = take(pace_table_bytes());
   L.partial = take((size_t)L.max_items * ebs * D * 4 * 2);
   L.total = off;
   return L;
@@ -410,6 +412,153 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   }
 }
 
+// Long sequences: the dQ dataflow in persistent waves with paced key positions (pace.h), one token per wave.
+template <typename T, int D> struct DqToken : SweepToken {
+  typename Elem<T>::v8 qf[D / 32], dof[D / 32];
+  f32x4 acc[D / 16];
+  float l2, dls;
+  int last_slot;
+  const T* kbase; const T* vbase;
+};
+
+template <typename T, int D, int BS>
+__global__ __launch_bounds__(256) void dq_sweep_kernel(DqParams p, PaceParams pp) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  using v4 = typename E::v4;
+  constexpr int NK = D / 32, NDT = D / 16, LD = lds_pitch(D);
+  __shared__ __attribute__((aligned(16))) T k_s[4][64][LD];
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lg = lane >> 4;
+  const int slot = (blockIdx.x >> 3) * 4 + wave;
+  const unsigned lane8 = lane * 8u;
+  T (*ks)[LD] = k_s[wave];
+  using Tok = DqToken<T, D>;
+  auto fetch = [&](int sw, Tok (&f)[1], int& reach) {
+    const SweepPlace sp = sweep_place(pp, sw, p.cu, p.batch, p.total_len);
+    reach = sp.reach;
+    const int h = sp.stream / p.GT, hq = (sp.stream % p.GT) * 16 + li;
+    const bool has_head = hq < p.G;
+    Tok& k = f[0];
+    const int t = sp.base + slot;
+    k.t = t <= sp.t_last ? t : -1;
+    k.my_blk = -1; k.todo = 0ull; k.e0 = 0;
+#pragma unroll
+    for (int i = 0; i < NDT; i++) k.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k.t < 0) return;
+    const int b = find_sequence(p.cu, p.batch, t);
+    const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
+    k.pos = t - s0; k.qb = k.pos / BS; k.last_slot = (len - 1) >> 5;
+    const int slot0 = seq_first_slot(p.cu, b);
+    k.kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D;
+    k.vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D;
+    k.ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
+    const int hh = h * p.G + (has_head ? hq : 0);
+    const T* qp = (const T*)p.q + (long long)t * p.qsn + (long long)hh * p.qsh + 8 * lg;
+    const T* dp_ = (const T*)p.dout + (long long)t * p.dsn + (long long)hh * p.dsh + 8 * lg;
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) {
+      k.qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+      k.dof[kk] = has_head ? ld16<v8>(dp_ + 32 * kk) : zero16<v8>();
+    }
+    k.my_blk = lane < p.topk ? k.ip[(long long)lane * p.isk] : -1;
+    k.l2 = has_head ? p.lse[(long long)hh * p.total_len + t] : INFINITY;
+    float dl;
+    if (p.o) {
+      const T* op_ = (const T*)p.o + (long long)t * p.osn + (long long)hh * p.osh + 8 * lg;
+      float part = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) {
+        const v8 of = has_head ? ld16<v8>(op_ + 32 * kk) : zero16<v8>();
+#pragma unroll
+        for (int e = 0; e < 8; e++) part = __builtin_fmaf((float)of[e], (float)k.dof[kk][e], part);
+      }
+      dl = column_sum(part);
+      if (has_head && lg == 0) p.delta[(long long)hh * p.total_len + t] = dl;
+    } else {
+      dl = has_head ? p.delta[(long long)hh * p.total_len + t] : 0.f;
+    }
+    k.dls = dl * p.sm_scale;
+    k.todo = __ballot(k.my_blk >= 0 && k.my_blk <= k.qb);
+  };
+  auto adopt = [&](Tok& k, const Tok& f, int) { k = f; };
+  auto visit = [&](Tok& k, int, int blk, auto after_loads) {
+#pragma unroll
+    for (int half = 0; half < (BS + 63) / 64; half++) {
+      const int key0 = blk * BS + 64 * half;
+      if (key0 > k.pos) break;
+      constexpr int NS = BS >= 64 ? 4 : BS / 16;
+      v8 kfr[NS][NK], vfr[NS][NK];
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++) {
+        const int st = min((key0 >> 4) + nt, 2 * k.last_slot + 1);
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) {
+          kfr[nt][kk] = ld16<v8>(k.kbase + (long long)(st * NK + kk) * 512 + lane8);
+          vfr[nt][kk] = ld16<v8>(k.vbase + (long long)(st * NK + kk) * 512 + lane8);
+        }
+      }
+      if (half == 0) after_loads();
+      f32x4 ds[NS];
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++) {
+        f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) {
+          st16(&ks[16 * nt + li][32 * kk + 8 * lg], kfr[nt][kk]);
+          s = E::mfma16(kfr[nt][kk], k.qf[kk], s);
+          dp = E::mfma16(vfr[nt][kk], k.dof[kk], dp);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          ds[nt][r] = fast_exp2(__builtin_fmaf(s[r], p.qk_scale, -k.l2)) * __builtin_fmaf(dp[r], p.sm_scale, -k.dls);
+      }
+      if (key0 + 16 * NS - 1 > k.pos) {
+#pragma unroll
+        for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (key0 + 16 * nt + 4 * lg + r > k.pos) ds[nt][r] = 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < (NS + 1) / 2; c++) {
+        v8 dsf;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          dsf[r] = (T)ds[2 * c][r];
+          dsf[4 + r] = (T)(2 * c + 1 < NS ? ds[(2 * c + 1) % NS][r] : 0.f);
+        }
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) {
+          const T* a0 = &ks[32 * c + 4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+          const T* a1 = &ks[32 * c + 16 + 4 * lg + (li >> 2)][16 * dt + 4 * (li & 3)];
+          s16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+          s16x4 y = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a1));
+          s16x8 z = {x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+          k.acc[dt] = E::mfma16(__builtin_bit_cast(v8, z), dsf, k.acc[dt]);
+        }
+      }
+    }
+  };
+  auto finish = [&](Tok& k, int, int sw) {
+    const int stream = sw / pp.sweeps_per_stream;
+    const int h = stream / p.GT, hq = (stream % p.GT) * 16 + li;
+    if (hq < p.G) {
+      T* op = (T*)p.dq + (long long)k.t * p.dqsn + (long long)(h * p.G + hq) * p.dqsh + 4 * lg;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        v4 out;
+#pragma unroll
+        for (int r = 0; r < 4; r++) out[r] = (T)k.acc[dt][r];
+        st8(op + 16 * dt, out);
+      }
+    }
+  };
+  run_paced_sweeps<BS, 1, false, Tok, Tok>(pp, p.topk, p.isk, lane, slot, fetch, adopt, visit, finish);
+}
+
 // ------------------------------------------------------------------------------------------
 struct BwdArgs {
   const void *q, *k, *v, *o, *dout; const float* lse; const int32_t* idx; const int32_t* cu; void *dq, *dk, *dv;
@@ -474,9 +623,18 @@ static int run_bwd(const BwdArgs& a) {
     p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
     p.sched = nsa_xcd_schedule(a.T, a.B, GT * (int)a.Hkv, (int)a.D, 8.0);
+    const bool paced = (a.phases & NSA_BWD_SCHEDULE_PACED) || (!(a.phases & NSA_BWD_SCHEDULE_PLAIN) && pace_pays(a.T, (int)a.D));
+    if (paced) {
+      PaceParams pace;
+      pace.table = (int32_t*)(ws + L.pace);
+      pace_fill_params(pace, a.T, pace_slots(), 1, pace_window_units((int)a.D));
+      launch_pace_prepare(pace, a.cu, (int)a.B, (int)a.T, GT * (int)a.Hkv, 2000, a.stream);
+      dq_sweep_kernel<T, D, BS><<<(unsigned)(2 * pace.slots), 256, 0, a.stream>>>(p, pace);
+    } else {
     long long n_wg = ((p.n_items + 3) / 4 + 7) / 8 * 8;
     if (p.sched.parts) n_wg = 8ll * p.sched.wgs_per_xcd;
     dq_kernel<T, D, BS><<<(unsigned)n_wg, 256, 0, a.stream>>>(p);
+    }
   }
   if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;

@@ -9,6 +9,7 @@
 // with one token per wave every K/V element feeds exactly one MFMA, so there is no reuse for
 // LDS to exploit.
 #include "retile.h"
+#include "pace.h"
 
 struct TopkFwdParams {
   const void* q; const void* kf; const void* vf; const int32_t* idx; void* o; float* lse; const int32_t* cu;
@@ -178,47 +179,229 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
 }
 
-template <typename T, int D, int BS>
-static int launch_fwd(const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn, long long vsh,
-                      int phases, hipStream_t stream) {
-  if (phases & NSA_FWD_PHASE_TRANSPOSE) {
-    launch_retile_pair<T, D, RETILE_ROWS, RETILE_COLS>((const T*)k, (T*)p.kf, ksn, ksh, (const T*)v, (T*)p.vf, vsn, vsh, p.cu, p.batch, p.n_slots, p.Hkv, stream);
+
+// ------------------------------------------------------------------------------------------
+// Long sequences: the same dataflow in persistent waves whose key positions are paced (pace.h).  A wave owns TPW
+// consecutive tokens of a sweep and visits the union of their selected blocks in ascending key order, one
+// (token, block) pair at a time; the per-token state (Q fragments, output accumulators, running maximum and sum)
+// stays in registers for the whole sweep.
+template <typename T, int D> struct FwdToken : SweepToken {
+  typename Elem<T>::v8 qf[D / 32];
+  f32x4 acc[D / 16];
+  float m, lsum;
+  int last_slot;
+  const T* kbase; const T* vbase;
+};
+// what a token brings with it: fetched one sweep ahead, so that the loads are long back when its turn comes
+template <typename T, int D> struct FwdAhead {
+  typename Elem<T>::v8 qf[D / 32];
+  int my_blk;
+  int t, pos, qb, last_slot;
+  const T* kbase; const T* vbase; const int32_t* ip;
+};
+
+// after_loads() runs once, after the fragment loads of the block's first slice have been issued
+template <typename T, int D, int BS, typename F>
+__device__ __forceinline__ void fwd_visit_block(FwdToken<T, D>& k, int blk, float qs, unsigned lane8, int lg, F after_loads) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  constexpr int NK = D / 32, NDT = D / 16;
+#pragma unroll
+  for (int sl = 0; sl < (BS + 63) / 64; sl++) {
+    const int key0 = blk * BS + 64 * sl;
+    if (key0 > k.pos) break;
+    constexpr int NS = BS >= 64 ? 4 : BS / 16, NC = NS / 2;
+    v8 kfr[NS][NK], vfr[NC][NDT];
+#pragma unroll
+    for (int nt = 0; nt < NS; nt++) {
+      const int st = min((key0 >> 4) + nt, 2 * k.last_slot + 1);
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) kfr[nt][kk] = ld16<v8>(k.kbase + (long long)(st * NK + kk) * 512 + lane8);
+    }
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+      const int slot = min((key0 >> 5) + c, k.last_slot);
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) vfr[c][dt] = ld16<v8>(k.vbase + (long long)slot * D * 32 + dt * 512 + lane8);
+    }
+    if (sl == 0) after_loads();
+    f32x4 s[NS];
+#pragma unroll
+    for (int nt = 0; nt < NS; nt++) {
+      f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) c = E::mfma16(kfr[nt][kk], k.qf[kk], c);
+      s[nt] = c;
+    }
+    if (key0 + 16 * NS - 1 > k.pos) {
+#pragma unroll
+      for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          if (key0 + 16 * nt + 4 * lg + r > k.pos) s[nt][r] = -INFINITY;
+    }
+    float mloc = M_FLOOR;
+#pragma unroll
+    for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) mloc = fmaxf(mloc, s[nt][r]);
+    mloc = column_max(mloc);
+    const bool moved = (mloc - k.m) * qs > RESCALE_SLACK;
+    if (__ballot(moved)) {
+      const float m_new = moved ? mloc : k.m;
+      const float alpha = fast_exp2((k.m - m_new) * qs);
+      k.m = m_new;
+      k.lsum *= alpha;
+#pragma unroll
+      for (int i = 0; i < NDT; i++) k.acc[i] *= alpha;
+    }
+    const float mb = k.m * qs;
+    float psum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const float x = fast_exp2(__builtin_fmaf(s[nt][r], qs, -mb));
+        s[nt][r] = x;
+        psum += x;
+      }
+    k.lsum += psum;
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+      v8 pf;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        pf[r] = (T)s[2 * c][r];
+        pf[4 + r] = (T)s[2 * c + 1][r];
+      }
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) k.acc[dt] = E::mfma16(vfr[c][dt], pf, k.acc[dt]);
+    }
   }
-  if (phases & NSA_FWD_PHASE_ATTEND) {
+}
+
+template <typename T, int D, int BS, int TPW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void topk_fwd_sweep_kernel(TopkFwdParams p, PaceParams pp) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  using v4 = typename E::v4;
+  constexpr int NK = D / 32, NDT = D / 16;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lg = lane >> 4;
+  const int slot = (blockIdx.x >> 3) * 4 + wave;
+  const unsigned lane8 = lane * 8u;
+  const float qs = fabsf(p.qk_scale);
+  using Tok = FwdToken<T, D>;
+  using Ahead = FwdAhead<T, D>;
+  auto fetch = [&](int sw, Ahead (&f)[TPW], int& reach) {
+    const SweepPlace sp = sweep_place(pp, sw, p.cu, p.batch, p.total_len);
+    reach = sp.reach;
+    const int h = sp.stream / p.GT, hq = (sp.stream % p.GT) * 16 + li;
+    const bool has_head = hq < p.G;
+#pragma unroll
+    for (int i = 0; i < TPW; i++) {
+      Ahead& k = f[i];
+      const int t = sp.base + slot * TPW + i;
+      k.t = t <= sp.t_last ? t : -1;
+      k.my_blk = -1;
+      if (k.t < 0) continue;
+      const int b = find_sequence(p.cu, p.batch, t);
+      const int s0 = p.cu[b], len = p.cu[b + 1] - s0;
+      k.pos = t - s0; k.qb = k.pos / BS; k.last_slot = (len - 1) >> 5;
+      const int slot0 = seq_first_slot(p.cu, b);
+      k.kbase = (const T*)p.kf + ((long long)h * p.n_slots + slot0) * 32 * D;
+      k.vbase = (const T*)p.vf + ((long long)h * p.n_slots + slot0) * 32 * D;
+      k.ip = p.idx + (long long)h * p.ish + (long long)t * p.isn;
+      const T* qp = (const T*)p.q + (long long)t * p.qsn + (long long)(h * p.G + (has_head ? hq : 0)) * p.qsh + 8 * lg;
+#pragma unroll
+      for (int kk = 0; kk < NK; kk++) k.qf[kk] = has_head ? ld16<v8>(qp + 32 * kk) : zero16<v8>();
+      k.my_blk = lane < p.topk ? k.ip[(long long)lane * p.isk] : -1;
+    }
+  };
+  auto adopt = [&](Tok& k, const Ahead& f, int) {
+    k.t = f.t; k.pos = f.pos; k.qb = f.qb; k.last_slot = f.last_slot; k.kbase = f.kbase; k.vbase = f.vbase; k.ip = f.ip;
+    k.my_blk = f.my_blk; k.e0 = 0; k.m = M_FLOOR; k.lsum = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < NK; kk++) k.qf[kk] = p.qk_scale < 0.f ? negated16(f.qf[kk]) : f.qf[kk];
+#pragma unroll
+    for (int d = 0; d < NDT; d++) k.acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    k.todo = k.t >= 0 ? __ballot(k.my_blk >= 0 && k.my_blk <= k.qb) : 0ull;
+  };
+  auto visit = [&](Tok& k, int, int blk, auto after_loads) { fwd_visit_block<T, D, BS>(k, blk, qs, lane8, lg, after_loads); };
+  auto finish = [&](Tok& k, int, int sw) {
+    const int stream = sw / pp.sweeps_per_stream;
+    const int h = stream / p.GT, hq = (stream % p.GT) * 16 + li;
+    const float lsum = column_sum(k.lsum);
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+    if (hq < p.G) {
+      T* op = (T*)p.o + (long long)k.t * p.osn + (long long)(h * p.G + hq) * p.osh + 4 * lg;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        v4 out;
+#pragma unroll
+        for (int r = 0; r < 4; r++) out[r] = (T)(k.acc[dt][r] * inv);
+        st8(op + 16 * dt, out);
+      }
+      if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + k.t] = lsum > 0.f ? k.m * qs + fast_log2(lsum) : -INFINITY;
+    }
+  };
+  run_paced_sweeps<BS, TPW, TPW == 1, Tok, Ahead>(pp, p.topk, p.isk, lane, slot, fetch, adopt, visit, finish);
+}
+
+// everything one forward call needs on the host side
+struct FwdCall {
+  TopkFwdParams p;
+  PaceParams pace;   // pace.slots == 0: the plain kernel
+  int tokens_per_wave, fixed_units;
+  const void* k; const void* v;
+  long long ksn, ksh, vsn, vsh;
+  int phases;
+  hipStream_t stream;
+};
+
+template <typename T, int D, int BS>
+static int launch_fwd(const FwdCall& c) {
+  const TopkFwdParams& p = c.p;
+  if (c.phases & NSA_FWD_PHASE_TRANSPOSE) {
+    launch_retile_pair<T, D, RETILE_ROWS, RETILE_COLS>((const T*)c.k, (T*)p.kf, c.ksn, c.ksh, (const T*)c.v, (T*)p.vf, c.vsn, c.vsh, p.cu, p.batch, p.n_slots, p.Hkv, c.stream);
+  }
+  if ((c.phases & NSA_FWD_PHASE_ATTEND) && c.pace.slots) {
+    launch_pace_prepare(c.pace, p.cu, p.batch, p.total_len, p.GT * p.Hkv, c.fixed_units, c.stream);
+    const unsigned n_wg = (unsigned)(2 * c.pace.slots);   // 8 XCDs x slots / 4 workgroups
+    topk_fwd_sweep_kernel<T, D, BS, 1><<<n_wg, 256, 0, c.stream>>>(p, c.pace);
+  } else if (c.phases & NSA_FWD_PHASE_ATTEND) {
     long long n_wg = (p.n_items + 3) / 4;
     n_wg = (n_wg + 7) / 8 * 8;
     if (p.sched.parts) n_wg = 8ll * p.sched.wgs_per_xcd;
-    topk_fwd_kernel<T, D, BS><<<dim3((unsigned)n_wg), 256, 0, stream>>>(p);
+    topk_fwd_kernel<T, D, BS><<<dim3((unsigned)n_wg), 256, 0, c.stream>>>(p);
   }
   return nsa_check_launch();
 }
 
 template <typename T, int D>
-static int dispatch_bs(int bs, const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn, long long vsh,
-                       int ph, hipStream_t s) {
+static int dispatch_bs(int bs, const FwdCall& c) {
   switch (bs) {
-    case 32: return launch_fwd<T, D, 32>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
-    case 64: return launch_fwd<T, D, 64>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
-    case 128: return launch_fwd<T, D, 128>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
-    case 256: return launch_fwd<T, D, 256>(p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 32: return launch_fwd<T, D, 32>(c);
+    case 64: return launch_fwd<T, D, 64>(c);
+    case 128: return launch_fwd<T, D, 128>(c);
+    case 256: return launch_fwd<T, D, 256>(c);
   }
   return NSA_ERR_UNSUPPORTED;
 }
 
 template <typename T>
-static int dispatch_d(int d, int bs, const TopkFwdParams& p, const void* k, long long ksn, long long ksh, const void* v, long long vsn,
-                      long long vsh, int ph, hipStream_t s) {
+static int dispatch_d(int d, int bs, const FwdCall& c) {
   switch (d) {
-    case 32: return dispatch_bs<T, 32>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
-    case 64: return dispatch_bs<T, 64>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
-    case 96: return dispatch_bs<T, 96>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
-    case 128: return dispatch_bs<T, 128>(bs, p, k, ksn, ksh, v, vsn, vsh, ph, s);
+    case 32: return dispatch_bs<T, 32>(bs, c);
+    case 64: return dispatch_bs<T, 64>(bs, c);
+    case 96: return dispatch_bs<T, 96>(bs, c);
+    case 128: return dispatch_bs<T, 128>(bs, c);
   }
   return NSA_ERR_UNSUPPORTED;
 }
 
 extern "C" size_t nsa_topk_attn_fwd_workspace_bytes(int64_t total_len, int64_t batch, int64_t num_kv_heads, int64_t head_dim) {
-  return 2 * retile_bytes(total_len, batch, num_kv_heads, head_dim);  // K and V copies
+  return 2 * retile_bytes(total_len, batch, num_kv_heads, head_dim) + pace_table_bytes();  // K and V copies, pacing table
 }
 
 extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t* topk_idx, void* o, float* lse,
@@ -237,8 +420,10 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   if ((o_stride_n | o_stride_h) % 4 != 0) return NSA_ERR_UNSUPPORTED;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)workspace) % 16 != 0 || (uintptr_t)o % 8 != 0) return NSA_ERR_UNSUPPORTED;
   if (workspace_bytes < nsa_topk_attn_fwd_workspace_bytes(total_len, batch, num_kv_heads, head_dim)) return NSA_ERR_WORKSPACE;
-  TopkFwdParams p;
-  p.q = q; p.kf = workspace; p.vf = (char*)workspace + retile_bytes(total_len, batch, num_kv_heads, head_dim); p.idx = topk_idx; p.o = o; p.lse = lse; p.cu = cu_seqlens;
+  FwdCall c;
+  TopkFwdParams& p = c.p;
+  const size_t copy_bytes = retile_bytes(total_len, batch, num_kv_heads, head_dim);
+  p.q = q; p.kf = workspace; p.vf = (char*)workspace + copy_bytes; p.idx = topk_idx; p.o = o; p.lse = lse; p.cu = cu_seqlens;
   p.total_len = (int)total_len; p.batch = (int)batch; p.Hkv = (int)num_kv_heads; p.G = (int)(num_q_heads / num_kv_heads);
   p.GT = (p.G + 15) / 16; p.topk = (int)topk; p.n_slots = (int)nsa_chunk_slots(total_len, batch);
   p.n_items = (long long)total_len * p.GT * p.Hkv;
@@ -248,9 +433,16 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   // a zero scale is applied as the smallest positive one: finite scores then still give probability 1, masked
   // (-inf) scores still probability 0 (with an exact zero they would give 0 * inf)
   p.qk_scale = (sm_scale == 0.f ? 1.17549435e-38f : sm_scale) * NSA_LOG2E;
-  hipStream_t s = (hipStream_t)stream;
-  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, p, k, k_stride_n, k_stride_h, v, v_stride_n, v_stride_h, phases, s);
-  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, p, k, k_stride_n, k_stride_h, v, v_stride_n, v_stride_h, phases, s);
+  c.k = k; c.v = v; c.ksn = k_stride_n; c.ksh = k_stride_h; c.vsn = v_stride_n; c.vsh = v_stride_h; c.phases = phases;
+  c.stream = (hipStream_t)stream;
+  c.pace.slots = 0; c.pace.table = (int32_t*)((char*)workspace + 2 * copy_bytes); c.tokens_per_wave = 1;
+  // fixed part of a sweep's cost in the XCD schedule, in 64-key positions: fitted to the per-XCD times of paced
+  // launches at 32 K .. 128 K tokens (1300 balances 32 K, 2500 the longer ones)
+  c.fixed_units = 2000;
+  const bool paced = (phases & NSA_FWD_SCHEDULE_PACED) || (!(phases & NSA_FWD_SCHEDULE_PLAIN) && pace_pays(total_len, (int)head_dim));
+  if (paced) pace_fill_params(c.pace, total_len, pace_slots(), c.tokens_per_wave, pace_window_units((int)head_dim));
+  if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, c);
+  if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, c);
   return NSA_ERR_UNSUPPORTED;
 }
 
