@@ -39,7 +39,8 @@ int nsa_version(void);
  * Forward: replaces forward_kernel launched from _topk_sparse_attention_fwd
  * (native_sparse_attention/ops/triton/topk_sparse_attention.py:828-909).
  *   q,o [T,Hq,D]; k,v [T,Hkv,D]; topk_idx int32 [Hkv,T,topk] (entries <0 or beyond the
- *   query's own block are skipped); lse fp32 [Hq,T] in base-2 units (contiguous).
+ *   query's own block are skipped; the ids of a row are a set: a block listed twice is attended
+ *   to once, here and in every pass of the backward); lse fp32 [Hq,T] in base-2 units (contiguous).
  * workspace holds fragment-major copies of K and V (2x their size) and a 16 KiB pacing table:
  * nsa_topk_attn_fwd_workspace_bytes().
  * phases: NSA_FWD_PHASE_ALL, or a subset when the caller re-uses the workspace of a previous

@@ -227,6 +227,26 @@ __device__ __forceinline__ int find_sequence(const int32_t* __restrict__ cu, int
   return lo;
 }
 
+// A token's row of selected block ids is a set: an id listed twice counts once (in the forward, in dQ and in the
+// reverse index alike).  The query-stationary kernels hold a stretch of 64 entries one per lane and visit the valid
+// ones through a bit mask.  row_stretch loads the stretch that starts at entry e0 into my_blk and returns the mask of
+// entries that are valid (0 <= id <= own block) and repeat no entry of an earlier stretch; repeats inside the stretch
+// are dropped when the first of them is visited (row_visited).
+__device__ __forceinline__ unsigned long long row_stretch(const int32_t* __restrict__ ip, long long isk, int topk, int e0, int lane, int own_block, int& my_blk) {
+  my_blk = e0 + lane < topk ? ip[(long long)(e0 + lane) * isk] : -1;
+  unsigned long long valid = __ballot(my_blk >= 0 && my_blk <= own_block);
+  for (int p0 = 0; p0 < e0 && valid; p0 += 64) {   // rows of more than 64 entries only
+    const int earlier = ip[(long long)(p0 + lane) * isk];
+    for (int j = 0; j < 64; j++) {
+      const int b = __builtin_amdgcn_readlane(earlier, j);
+      if (b >= 0) valid &= ~__ballot(my_blk == b);
+    }
+  }
+  return valid;
+}
+// mask of the entries still to visit once block blk has been taken
+__device__ __forceinline__ unsigned long long row_visited(unsigned long long todo, int my_blk, int blk) { return todo & ~__ballot(my_blk == blk); }
+
 // Spread consecutive logical work ids over the 8 XCDs in contiguous runs: hardware hands
 // workgroup i to XCD i%8, so logical id = (i%8)*ceil(n/8) + i/8 keeps neighbours on one L2.
 __device__ __forceinline__ long long xcd_remap(long long wg, long long n_wg) {

@@ -149,7 +149,7 @@ struct SweepToken {
 //   fetch(sw, ahead, reach)  loads what the tokens of sweep sw bring with them (AHEAD: one sweep early) and returns
 //                            the number of 64-key positions the sweep can reach;
 //   adopt(tok, ahead, i)     makes token i current (accumulators zeroed, todo set);
-//   visit(tok, i, blk, f)    one (token, block) pair; calls f() once its loads are issued;
+//   visit(tok, who, blk, f)  block blk for the tokens in the bit set who; calls f() once the block's loads are issued;
 //   finish(tok, i, sw)       writes the token's results.
 template <int BS, int TPW, bool AHEAD, typename Tok, typename Ahead, typename Fetch, typename Adopt, typename Visit, typename Finish>
 __device__ __forceinline__ void run_paced_sweeps(const PaceParams& pp, int topk, long long isk, int lane, int slot,
@@ -170,40 +170,49 @@ __device__ __forceinline__ void run_paced_sweeps(const PaceParams& pp, int topk,
 #pragma unroll
     for (int i = 0; i < TPW; i++) adopt(tok[i], ahead[i], i);
     if (AHEAD && sw + 1 < sw_end) fetch(sw + 1, ahead, reach_ahead);
-    // the (token, block) pair with the lowest key position among the wave's tokens, or sel < 0
-    auto next_pair = [&](int& sel, int& blk) {
-      sel = -1; blk = 0x7fffffff;
+    // the lowest block any of the wave's tokens has left, and the tokens (bit i: token i) of one sequence that are
+    // at it: they are served by one fetch of the block
+    auto next_pick = [&](unsigned& who, int& blk) {
+      who = 0u; blk = 0x7fffffff;
+      int at[TPW];
 #pragma unroll
       for (int i = 0; i < TPW; i++) {
         SweepToken& k = tok[i];
+        at[i] = 0x7fffffff;
         if (k.t < 0) continue;
         while (!k.todo && k.e0 + 64 < topk) {   // rows longer than 64 entries: next stretch
           k.e0 += 64;
-          k.my_blk = k.e0 + lane < topk ? k.ip[(long long)(k.e0 + lane) * isk] : -1;
-          k.todo = __ballot(k.my_blk >= 0 && k.my_blk <= k.qb);
+          k.todo = row_stretch(k.ip, isk, topk, k.e0, lane, k.qb, k.my_blk);
         }
-        if (!k.todo) continue;
-        const int b = __builtin_amdgcn_readlane(k.my_blk, __builtin_ctzll(k.todo));
-        if (b < blk) { blk = b; sel = i; }
+        if (k.todo) at[i] = __builtin_amdgcn_readlane(k.my_blk, __builtin_ctzll(k.todo));
+        blk = min(blk, at[i]);
       }
-    };
-    int sel, blk;
-    next_pair(sel, blk);
-    int position = sel >= 0 ? origin + ((blk * BS) >> 6) : origin + reach;
-    pc.publish(position);
-    while (sel >= 0) {
-      pc.wait(position);
-      int sel_next = -1, blk_next = 0;
+      if (blk == 0x7fffffff) return;
+      int seq_start = 0;
 #pragma unroll
       for (int i = 0; i < TPW; i++) {
-        if (sel != i) continue;
-        tok[i].todo &= tok[i].todo - 1;
-        next_pair(sel_next, blk_next);
-        position = sel_next >= 0 ? origin + ((blk_next * BS) >> 6) : origin + reach;
-        // once this pair's loads are on their way the wave no longer needs the L2 to hold its lines
-        visit(tok[i], i, blk, [&] { pc.publish(position); });
+        if (at[i] != blk) continue;
+        if (!who) seq_start = tok[i].t - tok[i].pos;
+        if (tok[i].t - tok[i].pos == seq_start) who |= 1u << i;
       }
-      sel = sel_next; blk = blk_next;
+    };
+    unsigned who;
+    int blk;
+    next_pick(who, blk);
+    int position = who ? origin + ((blk * BS) >> 6) : origin + reach;
+    pc.publish(position);
+    while (who) {
+      pc.wait(position);
+#pragma unroll
+      for (int i = 0; i < TPW; i++)
+        if (who >> i & 1) tok[i].todo = row_visited(tok[i].todo, tok[i].my_blk, blk);
+      unsigned who_next;
+      int blk_next;
+      next_pick(who_next, blk_next);
+      position = who_next ? origin + ((blk_next * BS) >> 6) : origin + reach;
+      // once this block's loads are on their way the wave no longer needs the L2 to hold its lines
+      visit(tok, who, blk, [&] { pc.publish(position); });
+      who = who_next; blk = blk_next;
     }
     origin += reach;
 #pragma unroll

@@ -333,13 +333,11 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   const int last_slot = (len - 1) >> 5;
   // block ids are read once (lane e holds entry e) and visited through a wave-uniform bit mask
   for (int e0 = 0; e0 < p.topk; e0 += 64) {
-  const int my_e = e0 + lane;
-  const int my_blk = my_e < p.topk ? ip[(long long)my_e * p.isk] : -1;
-  unsigned long long todo = __ballot(my_blk >= 0 && my_blk <= qb);
+  int my_blk;
+  unsigned long long todo = row_stretch(ip, p.isk, p.topk, e0, lane, qb, my_blk);
   while (todo) {
-    const int e = __builtin_ctzll(todo);
-    todo &= todo - 1;
-    const int blk = __builtin_amdgcn_readlane(my_blk, e);
+    const int blk = __builtin_amdgcn_readlane(my_blk, __builtin_ctzll(todo));
+    todo = row_visited(todo, my_blk, blk);
     // 64 keys at a time (larger blocks are walked in 64-key slices); all fragment loads of a slice
     // are issued back to back before any of them is consumed
 #pragma unroll
@@ -484,7 +482,8 @@ __global__ __launch_bounds__(256) void dq_sweep_kernel(DqParams p, PaceParams pp
     k.todo = __ballot(k.my_blk >= 0 && k.my_blk <= k.qb);
   };
   auto adopt = [&](Tok& k, const Tok& f, int) { k = f; };
-  auto visit = [&](Tok& k, int, int blk, auto after_loads) {
+  auto visit = [&](Tok (&tok)[1], unsigned, int blk, auto after_loads) {
+    Tok& k = tok[0];
 #pragma unroll
     for (int half = 0; half < (BS + 63) / 64; half++) {
       const int key0 = blk * BS + 64 * half;

@@ -76,13 +76,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // the row of block ids is read once, 64 entries at a time (lane e holds entry e); the valid
   // ones are then visited through a wave-uniform bit mask, so no load sits between two blocks
   for (int e0 = 0; e0 < p.topk; e0 += 64) {
-  const int my_e = e0 + lane;
-  const int my_blk = my_e < p.topk ? ip[(long long)my_e * p.isk] : -1;
-  unsigned long long todo = __ballot(my_blk >= 0 && my_blk <= qb);
+  int my_blk;
+  unsigned long long todo = row_stretch(ip, p.isk, p.topk, e0, lane, qb, my_blk);
   while (todo) {
-    const int e = __builtin_ctzll(todo);
-    todo &= todo - 1;
-    const int blk = __builtin_amdgcn_readlane(my_blk, e);
+    const int blk = __builtin_amdgcn_readlane(my_blk, __builtin_ctzll(todo));
+    todo = row_visited(todo, my_blk, blk);
     // a block is walked in slices of up to 64 keys: all 2*NS*NK + NC*NDT fragment loads of a slice
     // are issued back to back (no branches in between) so that ~32 KiB per wave are in flight
 #pragma unroll
@@ -182,9 +180,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 // ------------------------------------------------------------------------------------------
 // Long sequences: the same dataflow in persistent waves whose key positions are paced (pace.h).  A wave owns TPW
-// consecutive tokens of a sweep and visits the union of their selected blocks in ascending key order, one
-// (token, block) pair at a time; the per-token state (Q fragments, output accumulators, running maximum and sum)
-// stays in registers for the whole sweep.
+// consecutive tokens of a sweep and visits the union of their selected blocks in ascending key order; the per-token
+// state (Q fragments, output accumulators, running maximum and sum) stays in registers for the whole sweep.  Only
+// TPW = 1 is launched: with two tokens per wave (a block that both select is fetched once, half as many sweeps
+// stream the prefix) the state no longer fits 256 registers beside the 128 of a block in flight, and the spills cost
+// more than the sharing saves (forward at 32 K / 64 K / 128 K tokens: 2.84 / 6.14 / 14.9 ms against 2.75 / 5.74 / 13.9).
 template <typename T, int D> struct FwdToken : SweepToken {
   typename Elem<T>::v8 qf[D / 32];
   f32x4 acc[D / 16];
@@ -200,82 +200,98 @@ template <typename T, int D> struct FwdAhead {
   const T* kbase; const T* vbase; const int32_t* ip;
 };
 
-// after_loads() runs once, after the fragment loads of the block's first slice have been issued
-template <typename T, int D, int BS, typename F>
-__device__ __forceinline__ void fwd_visit_block(FwdToken<T, D>& k, int blk, float qs, unsigned lane8, int lg, F after_loads) {
+// One block for the tokens of `who` (all of one sequence): the K/V fragments of a slice are fetched once and serve
+// every token of the set.  after_loads() runs once, after the fragment loads of the block's first slice have been issued.
+template <typename T, int D, int BS, int TPW, typename F>
+__device__ __forceinline__ void fwd_visit_block(FwdToken<T, D> (&tok)[TPW], unsigned who, int blk, float qs, unsigned lane8, int lg, F after_loads) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   constexpr int NK = D / 32, NDT = D / 16;
+  int first = 0, pos_max = -1;
+#pragma unroll
+  for (int i = TPW - 1; i >= 0; i--)
+    if (who >> i & 1) { first = i; pos_max = max(pos_max, tok[i].pos); }
+  const T* kbase = tok[0].kbase; const T* vbase = tok[0].vbase;
+  int last_slot = tok[0].last_slot;
+#pragma unroll
+  for (int i = 1; i < TPW; i++)
+    if (first == i) { kbase = tok[i].kbase; vbase = tok[i].vbase; last_slot = tok[i].last_slot; }
 #pragma unroll
   for (int sl = 0; sl < (BS + 63) / 64; sl++) {
     const int key0 = blk * BS + 64 * sl;
-    if (key0 > k.pos) break;
+    if (key0 > pos_max) break;
     constexpr int NS = BS >= 64 ? 4 : BS / 16, NC = NS / 2;
     v8 kfr[NS][NK], vfr[NC][NDT];
 #pragma unroll
     for (int nt = 0; nt < NS; nt++) {
-      const int st = min((key0 >> 4) + nt, 2 * k.last_slot + 1);
+      const int st = min((key0 >> 4) + nt, 2 * last_slot + 1);   // sub-tiles wholly in the future: clamp onto storage that exists
 #pragma unroll
-      for (int kk = 0; kk < NK; kk++) kfr[nt][kk] = ld16<v8>(k.kbase + (long long)(st * NK + kk) * 512 + lane8);
+      for (int kk = 0; kk < NK; kk++) kfr[nt][kk] = ld16<v8>(kbase + (long long)(st * NK + kk) * 512 + lane8);
     }
 #pragma unroll
     for (int c = 0; c < NC; c++) {
-      const int slot = min((key0 >> 5) + c, k.last_slot);
+      const int slot = min((key0 >> 5) + c, last_slot);
 #pragma unroll
-      for (int dt = 0; dt < NDT; dt++) vfr[c][dt] = ld16<v8>(k.vbase + (long long)slot * D * 32 + dt * 512 + lane8);
+      for (int dt = 0; dt < NDT; dt++) vfr[c][dt] = ld16<v8>(vbase + (long long)slot * D * 32 + dt * 512 + lane8);
     }
     if (sl == 0) after_loads();
-    f32x4 s[NS];
 #pragma unroll
-    for (int nt = 0; nt < NS; nt++) {
-      f32x4 c = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < TPW; i++) {
+      FwdToken<T, D>& k = tok[i];
+      if (!(who >> i & 1) || key0 > k.pos) continue;
+      f32x4 s[NS];
 #pragma unroll
-      for (int kk = 0; kk < NK; kk++) c = E::mfma16(kfr[nt][kk], k.qf[kk], c);
-      s[nt] = c;
-    }
-    if (key0 + 16 * NS - 1 > k.pos) {
+      for (int nt = 0; nt < NS; nt++) {
+        f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; kk++) c = E::mfma16(kfr[nt][kk], k.qf[kk], c);
+        s[nt] = c;
+      }
+      // only the slice that holds the query's own position needs the causal test
+      if (key0 + 16 * NS - 1 > k.pos) {
+#pragma unroll
+        for (int nt = 0; nt < NS; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (key0 + 16 * nt + 4 * lg + r > k.pos) s[nt][r] = -INFINITY;
+      }
+      float mloc = M_FLOOR;
 #pragma unroll
       for (int nt = 0; nt < NS; nt++)
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-          if (key0 + 16 * nt + 4 * lg + r > k.pos) s[nt][r] = -INFINITY;
-    }
-    float mloc = M_FLOOR;
+        for (int r = 0; r < 4; r++) mloc = fmaxf(mloc, s[nt][r]);
+      mloc = column_max(mloc);
+      const bool moved = (mloc - k.m) * qs > RESCALE_SLACK;
+      if (__ballot(moved)) {
+        const float m_new = moved ? mloc : k.m;
+        const float alpha = fast_exp2((k.m - m_new) * qs);
+        k.m = m_new;
+        k.lsum *= alpha;
 #pragma unroll
-    for (int nt = 0; nt < NS; nt++)
-#pragma unroll
-      for (int r = 0; r < 4; r++) mloc = fmaxf(mloc, s[nt][r]);
-    mloc = column_max(mloc);
-    const bool moved = (mloc - k.m) * qs > RESCALE_SLACK;
-    if (__ballot(moved)) {
-      const float m_new = moved ? mloc : k.m;
-      const float alpha = fast_exp2((k.m - m_new) * qs);
-      k.m = m_new;
-      k.lsum *= alpha;
-#pragma unroll
-      for (int i = 0; i < NDT; i++) k.acc[i] *= alpha;
-    }
-    const float mb = k.m * qs;
-    float psum = 0.f;
-#pragma unroll
-    for (int nt = 0; nt < NS; nt++)
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const float x = fast_exp2(__builtin_fmaf(s[nt][r], qs, -mb));
-        s[nt][r] = x;
-        psum += x;
+        for (int d = 0; d < NDT; d++) k.acc[d] *= alpha;
       }
-    k.lsum += psum;
+      const float mb = k.m * qs;
+      float psum = 0.f;
 #pragma unroll
-    for (int c = 0; c < NC; c++) {
-      v8 pf;
+      for (int nt = 0; nt < NS; nt++)
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        pf[r] = (T)s[2 * c][r];
-        pf[4 + r] = (T)s[2 * c + 1][r];
+        for (int r = 0; r < 4; r++) {
+          const float x = fast_exp2(__builtin_fmaf(s[nt][r], qs, -mb));
+          s[nt][r] = x;
+          psum += x;
+        }
+      k.lsum += psum;
+#pragma unroll
+      for (int c = 0; c < NC; c++) {
+        v8 pf;  // probabilities of masked keys are exactly 0, the clamped V data they meet is finite
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          pf[r] = (T)s[2 * c][r];
+          pf[4 + r] = (T)s[2 * c + 1][r];
+        }
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) k.acc[dt] = E::mfma16(vfr[c][dt], pf, k.acc[dt]);
       }
-#pragma unroll
-      for (int dt = 0; dt < NDT; dt++) k.acc[dt] = E::mfma16(vfr[c][dt], pf, k.acc[dt]);
     }
   }
 }
@@ -327,7 +343,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int d = 0; d < NDT; d++) k.acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
     k.todo = k.t >= 0 ? __ballot(k.my_blk >= 0 && k.my_blk <= k.qb) : 0ull;
   };
-  auto visit = [&](Tok& k, int, int blk, auto after_loads) { fwd_visit_block<T, D, BS>(k, blk, qs, lane8, lg, after_loads); };
+  auto visit = [&](Tok (&tok)[TPW], unsigned who, int blk, auto after_loads) { fwd_visit_block<T, D, BS, TPW>(tok, who, blk, qs, lane8, lg, after_loads); };
   auto finish = [&](Tok& k, int, int sw) {
     const int stream = sw / pp.sweeps_per_stream;
     const int h = stream / p.GT, hq = (stream % p.GT) * 16 + li;

@@ -4,14 +4,19 @@ MAX_ABS, MEAN_ABS = 2e-2, 2e-3   # bf16/fp16 inputs, fp32 accumulation
 
 
 def assert_close(got: torch.Tensor, want: torch.Tensor, what: str, max_abs: float = MAX_ABS, mean_abs: float = MEAN_ABS, rel_to=None):
-    """max-abs / mean-abs bound; for gradients whose magnitude is far from 1 pass rel_to to scale the bound."""
+    """max-abs / mean-abs bound against the oracle.  Plain (rel_to None): absolute bounds, for outputs of magnitude ~1.
+    With rel_to (any value): every row (last dimension: the head_dim values of one token and head, the taps of one
+    pooling weight ...) is held to the bounds scaled by max(1, largest reference magnitude of THAT row) - gradients of
+    early keys sum over thousands of queries and reach the hundreds, where half a bf16 ulp alone is 0.1, while late keys
+    and most query rows stay below 1 and are held to the absolute bound."""
     g, w = got.float(), want.float()
     assert g.shape == w.shape, (what, g.shape, w.shape)
     assert torch.isfinite(g).all(), what + ": non-finite values"
-    scale = 1.0 if rel_to is None else max(1.0, float(rel_to))
     err = (g - w).abs()
-    assert err.max().item() <= max_abs * scale, "%s: max abs err %.4g > %.4g" % (what, err.max().item(), max_abs * scale)
-    assert err.mean().item() <= mean_abs * scale, "%s: mean abs err %.4g > %.4g" % (what, err.mean().item(), mean_abs * scale)
+    if rel_to is not None and w.dim() >= 1 and w.numel() > 0:
+        err = err / w.abs().amax(dim=-1, keepdim=True).clamp(min=1.0)
+    assert err.max().item() <= max_abs, "%s: max abs err %.4g (relative to its row's scale) > %.4g" % (what, err.max().item(), max_abs)
+    assert err.mean().item() <= mean_abs, "%s: mean abs err %.4g (relative to row scales) > %.4g" % (what, err.mean().item(), mean_abs)
 
 
 def clear_margin_rows(block_score: torch.Tensor, want_idx: torch.Tensor, q_block: torch.Tensor, margin: float = 1e-3) -> torch.Tensor:

@@ -93,6 +93,33 @@ def test_backward_matches_oracle(device, lens, Hq, Hkv, d, bs, topk, dtype, loca
     _grad_check(device, lens, Hq, Hkv, d, bs, topk, dtype, local)
 
 
+@pytest.mark.parametrize("schedule", [8, 16])   # NSA_*_SCHEDULE_PLAIN / _PACED
+def test_repeated_block_ids_count_once(device, schedule):
+    """A row that lists a block twice attends to it once (the ids of a row are a set, as in the oracle's mask), in the
+    forward, dQ, dK and dV alike."""
+    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
+
+    lens, Hq, Hkv, d, bs, topk = [900, 1300], 16, 2, 64, 64, 6
+    q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device, seed=3)
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=7)
+    rep = idx.clone()
+    rows = (idx[..., 3] >= 0)                       # rows with at least four valid entries
+    rep[..., 2] = torch.where(rows, idx[..., 1], idx[..., 2])   # entry 2 repeats entry 1 (block idx[..., 2] is dropped)
+    rep[..., 4] = torch.where(rows & (idx[..., 4] >= 0), idx[..., 0], idx[..., 4])   # a repeat that is not adjacent
+    assert int((rep != idx).sum()) > 1000
+    g = torch.Generator(device=device).manual_seed(11)
+    do = torch.randn(q.shape, generator=g, device=device).to(q.dtype)
+    n, sm = max(lens), d ** -0.5
+    o, lse = _topk_sparse_attention_fwd(q, k, v, rep, bs, cu, cu, n, n, sm, phases=3 | schedule)
+    dq, dk, dv = _topk_sparse_attention_bwd(o, do, lse, q, k, v, rep, bs, cu, cu, n, n, sm, phases=7 | schedule)
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, k, v))
+    want = oracle.topk_sparse_attention(qf, kf, vf, rep, bs, cu)
+    want.backward(do.float())
+    assert_close(o, want, "o")
+    for name, got, ref in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        assert_close(got, ref, name, rel_to=ref.abs().max().item())
+
+
 def _expand_to_pieces(idx, cu, bs, piece):
     """Ids of the `piece`-key pieces of the selected bs-key blocks that start at or before each token (-1 elsewhere)."""
     sub = bs // piece
@@ -190,5 +217,13 @@ def test_any_finite_softmax_scale(device, scale):
     do = torch.randn_like(o)
     o.backward(do)
     want.backward(do.float())
+    # At scale 3 the softmax is nearly one-hot and dS = scale * P * (dP - delta) is a difference of nearly equal numbers
+    # times 3: delta is formed from the 16-bit O (as the reference's backward_sum_o_do does, topk_sparse_attention.py:177-217),
+    # whose rounding (2^-9 of |o| per element, summed over d with |dO| ~ 1) alone moves dS by ~0.1.  That case is a test of
+    # "any finite scale runs and stays close", with the bounds scaled by the largest gradient; the others use row scales.
     for name, a, b in (("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)):
-        assert_close(a, b, name, rel_to=max(1.0, b.abs().max().item()))
+        if scale == 3.0:
+            s_ = max(1.0, b.abs().max().item())
+            assert_close(a, b, name, max_abs=2e-2 * s_, mean_abs=2e-3 * s_)
+        else:
+            assert_close(a, b, name, rel_to=True)
