@@ -15,11 +15,14 @@ struct RopeParams {
   int inverse;
 };
 
-template <typename T, int D>
-__global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
-  using v8 = typename Elem<T>::v8;
-  constexpr int HALF = D / 2, VEC = HALF / 8;  // 8-element pieces per half row
-  __shared__ float cos_s[HALF], sin_s[HALF];
+// V: elements per load/store piece (8 when half a row is a multiple of 8 elements, else 4); any head_dim that is a
+// multiple of 8 up to 2 * ROPE_MAX_HALF runs.
+constexpr int ROPE_MAX_HALF = 128;
+template <typename T, int V>
+__global__ __launch_bounds__(256) void rope_kernel(RopeParams p, int D) {
+  typedef T vec __attribute__((ext_vector_type(V)));
+  const int HALF = D / 2, VEC = HALF / V;  // V-element pieces per half row
+  __shared__ float cos_s[ROPE_MAX_HALF], sin_s[ROPE_MAX_HALF];
   const int n = blockIdx.x;
   int pos;
   if (p.step < 0) {   // the caller supplies one position index per row
@@ -40,30 +43,26 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
   const T* xr = (const T*)p.x + (long long)n * p.xsn;
   T* orow = (T*)p.out + (long long)n * p.osn;
   for (int i = threadIdx.x; i < p.H * VEC; i += 256) {
-    const int h = i / VEC, c8 = (i % VEC) * 8;
-    const v8 x1 = ld16<v8>(xr + (long long)h * p.xsh + c8), x2 = ld16<v8>(xr + (long long)h * p.xsh + HALF + c8);
-    v8 o1, o2;
+    const int h = i / VEC, c8 = (i % VEC) * V;
+    const vec x1 = *reinterpret_cast<const vec*>(xr + (long long)h * p.xsh + c8), x2 = *reinterpret_cast<const vec*>(xr + (long long)h * p.xsh + HALF + c8);
+    vec o1, o2;
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
+    for (int e = 0; e < V; e++) {
       const float c = cos_s[c8 + e], s = sin_s[c8 + e];
       const float a1 = (float)x1[e], a2 = (float)x2[e];
       o1[e] = (T)(rounded<T>(a1 * c) - rounded<T>(a2 * s));
       o2[e] = (T)(rounded<T>(a2 * c) + rounded<T>(a1 * s));
     }
-    st16(orow + (long long)h * p.osh + c8, o1);
-    st16(orow + (long long)h * p.osh + HALF + c8, o2);
+    *reinterpret_cast<vec*>(orow + (long long)h * p.osh + c8) = o1;
+    *reinterpret_cast<vec*>(orow + (long long)h * p.osh + HALF + c8) = o2;
   }
 }
 
 template <typename T>
 static int rope_dispatch(const RopeParams& p, int d, hipStream_t s) {
-  switch (d) {
-    case 32: rope_kernel<T, 32><<<p.n_rows, 256, 0, s>>>(p); break;
-    case 64: rope_kernel<T, 64><<<p.n_rows, 256, 0, s>>>(p); break;
-    case 96: rope_kernel<T, 96><<<p.n_rows, 256, 0, s>>>(p); break;
-    case 128: rope_kernel<T, 128><<<p.n_rows, 256, 0, s>>>(p); break;
-    default: return NSA_ERR_UNSUPPORTED;
-  }
+  if (d <= 0 || d % 8 != 0 || d > 2 * ROPE_MAX_HALF) return NSA_ERR_UNSUPPORTED;
+  if (d % 16 == 0) rope_kernel<T, 8><<<p.n_rows, 256, 0, s>>>(p, d);
+  else rope_kernel<T, 4><<<p.n_rows, 256, 0, s>>>(p, d);
   return nsa_check_launch();
 }
 
@@ -74,7 +73,9 @@ extern "C" int nsa_rope(const void* x, void* out, const float* inv_freq, const i
   if (!x || !out || !inv_freq || !cu_seqlens) return NSA_ERR_BAD_ARG;
   if (n_rows < 0 || batch <= 0 || num_heads <= 0 || stride <= 0 || n_rows >= (1ll << 31)) return NSA_ERR_BAD_ARG;
   if (step > 0 && n_rows != batch) return NSA_ERR_BAD_ARG;
-  if ((x_stride_n | x_stride_h | o_stride_n | o_stride_h) % 8 != 0 || ((uintptr_t)x | (uintptr_t)out) % 16 != 0) return NSA_ERR_UNSUPPORTED;
+  // 16-byte pieces (8-byte ones when half a row is an odd multiple of 4 elements)
+  const int64_t piece = head_dim % 16 == 0 ? 8 : 4;
+  if ((x_stride_n | x_stride_h | o_stride_n | o_stride_h) % piece != 0 || ((uintptr_t)x | (uintptr_t)out) % (2 * piece) != 0) return NSA_ERR_UNSUPPORTED;
   if (n_rows == 0) return NSA_OK;
   RopeParams p;
   p.x = x; p.out = out; p.inv_freq = inv_freq; p.cu = cu_seqlens;

@@ -9,7 +9,7 @@ from typing import Optional, Tuple, Union
 import torch
 
 from .. import _lib
-from .utils import last_dim_contiguous
+from .utils import last_dim_contiguous, pad_head_dim
 
 
 def _compressed_attention_fwd(q, k, v, kernel_size, kernel_stride, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale):
@@ -121,17 +121,20 @@ def compressed_attention(
         max_seqlen_q = (cu_seqlens_q[1:] - cu_seqlens_q[:-1]).max().item()
     if max_seqlen_k is None:
         max_seqlen_k = (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).max().item()
+    d = q.shape[-1]
     if sm_scale is None:
-        sm_scale = 1 / math.sqrt(q.shape[-1])
+        sm_scale = 1 / math.sqrt(d)
+    q, k, v = pad_head_dim(q, k, v)
     attn_output, lse = CompressedAttention.apply(
         q, k, v, kernel_size, kernel_stride, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale)
+    out = attn_output if attn_output.shape[-1] == d else attn_output[..., :d].contiguous()
     if topk <= 0:
         warnings.warn("topk <= 0, returned topk_idx will be None")
-        return attn_output, None
+        return out, None
     assert topk >= init_blocks + local_blocks
     assert block_size % kernel_size == 0 and kernel_size % kernel_stride == 0
     with torch.no_grad():
         k_out = min(topk, math.ceil(max_seqlen_q / block_size))
         topk_idx = _select_blocks(q.detach(), k.detach(), lse, kernel_size, kernel_stride, block_size, k_out, cu_seqlens_q,
                                   cu_seqlens_k, max_seqlen_q, init_blocks, local_blocks, sm_scale)
-    return attn_output, topk_idx
+    return out, topk_idx

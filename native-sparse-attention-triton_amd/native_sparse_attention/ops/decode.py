@@ -9,7 +9,7 @@ from typing import Optional, Tuple
 import torch
 
 from .. import _lib
-from .utils import last_dim_contiguous
+from .utils import built_head_dim, last_dim_contiguous, pad_head_dim
 
 
 def _common_checks(q, k, v, seqlens):
@@ -41,6 +41,8 @@ def flash_attention_decode(q, k, v, seqlens, sm_scale: Optional[float] = None) -
     B, Hq, Hkv, D, L = _common_checks(q, k, v, seqlens)
     if sm_scale is None:
         sm_scale = 1 / math.sqrt(D)
+    if L > 0 and built_head_dim(D) != D:   # head size between the built ones: zero columns appended (copies the slabs)
+        return flash_attention_decode(*pad_head_dim(q, k, v), seqlens, sm_scale)[..., :D].contiguous()
     q, k, v = map(last_dim_contiguous, (q, k, v))
     o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     if L == 0:
@@ -62,6 +64,8 @@ def topk_sparse_attention_decode(q, k, v, topk_idx, block_size: int, seqlens, sm
     topk = topk_idx.shape[-1]
     if sm_scale is None:
         sm_scale = 1 / math.sqrt(D)
+    if L > 0 and topk > 0 and built_head_dim(D) != D:
+        return topk_sparse_attention_decode(*pad_head_dim(q, k, v), topk_idx, block_size, seqlens, sm_scale)[..., :D].contiguous()
     q, k, v = map(last_dim_contiguous, (q, k, v))
     o = torch.empty_like(q, memory_format=torch.contiguous_format)  # the merge kernel writes every element
     if L == 0 or topk == 0:
@@ -95,6 +99,10 @@ def compressed_attention_decode(
         sm_scale = 1.0 / math.sqrt(D)
     if L == 0:  # input too short to have a compressed token
         return torch.zeros_like(q), torch.zeros(Hkv, B, 1, device=q.device, dtype=torch.int32)
+    if built_head_dim(D) != D:
+        o, idx = compressed_attention_decode(*pad_head_dim(q, k, v), seqlens, compress_seqlens, kernel_size, kernel_stride, block_size,
+                                             topk, init_blocks, local_blocks, sm_scale, max_seqlen)
+        return o[..., :D].contiguous(), idx
     q, k, v = map(last_dim_contiguous, (q, k, v))
     if max_seqlen is None:
         max_seqlen = int(seqlens.max())  # fixes the output shape; the reference synchronises here too (:30)

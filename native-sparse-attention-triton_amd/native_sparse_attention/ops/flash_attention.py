@@ -6,7 +6,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from .utils import last_dim_contiguous
+from .utils import last_dim_contiguous, pad_head_dim
 
 
 def _flash_attention_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale, gqa_interleave=False):
@@ -76,8 +76,12 @@ def flash_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu
     assert cu_seqlens_q.dtype == torch.int32 and cu_seqlens_k.dtype == torch.int32 and cu_seqlens_q.shape == cu_seqlens_k.shape
     Hq, Hkv = q.shape[1], k.shape[1]
     assert k.shape == v.shape and q.shape[2] == k.shape[2] and Hq % Hkv == 0
+    d = q.shape[-1]
     if sm_scale is None:
-        sm_scale = 1 / math.sqrt(q.shape[-1])
+        sm_scale = 1 / math.sqrt(d)
+    if pad_head_dim(q)[0].shape[-1] != d:   # head size between the built ones: zero columns appended
+        o = flash_attention_varlen(*pad_head_dim(q, k, v), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale, gqa_interleave)
+        return o[..., :d].contiguous()
     if gqa_interleave and Hq != Hkv:
         G = Hq // Hkv
         # the kernels group G consecutive query heads per kv head: reorder (g, kv) -> (kv, g) and back

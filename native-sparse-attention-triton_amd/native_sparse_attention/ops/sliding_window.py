@@ -9,7 +9,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from .utils import last_dim_contiguous
+from .utils import last_dim_contiguous, pad_head_dim
 
 
 def _window_fwd(q, k, v, cu_seqlens, window_size, sm_scale):
@@ -66,6 +66,9 @@ def sliding_window_attention_varlen(q, k, v, cu_seqlens, window_size: int, sm_sc
     assert q.dtype == torch.bfloat16 or q.dtype == torch.float16
     assert k.dtype == q.dtype and v.dtype == q.dtype and cu_seqlens.dtype == torch.int32
     assert k.shape[0] == q.shape[0] and v.shape == k.shape and q.shape[1] % k.shape[1] == 0 and window_size >= 0
+    d = q.shape[-1]
     if sm_scale is None:
-        sm_scale = 1 / math.sqrt(q.shape[-1])
-    return SlidingWindowAttention.apply(q, k, v, cu_seqlens, int(window_size), float(sm_scale))
+        sm_scale = 1 / math.sqrt(d)
+    q, k, v = pad_head_dim(q, k, v)   # head size between the built ones: zero columns appended
+    o = SlidingWindowAttention.apply(q, k, v, cu_seqlens, int(window_size), float(sm_scale))
+    return o if o.shape[-1] == d else o[..., :d].contiguous()

@@ -6,6 +6,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
+from .utils import pad_head_dim
 
 
 def _last_dim_contiguous(t: torch.Tensor) -> torch.Tensor:
@@ -139,4 +140,9 @@ def topk_sparse_attention(
     The kernels walk the token range directly, so unlike the reference wrapper (:1205) no
     host synchronisation is needed to learn the longest sequence.
     """
-    return TopkSparseAttention.apply(q, k, v, topk_idx, block_size, cu_seqlens, cu_seqlens, None, None, softmax_scale)
+    d = q.shape[-1]
+    if softmax_scale is None:
+        softmax_scale = 1 / math.sqrt(d)
+    q, k, v = pad_head_dim(q, k, v)
+    o = TopkSparseAttention.apply(q, k, v, topk_idx, block_size, cu_seqlens, cu_seqlens, None, None, softmax_scale)
+    return o if o.shape[-1] == d else o[..., :d].contiguous()

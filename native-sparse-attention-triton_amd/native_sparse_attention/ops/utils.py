@@ -28,3 +28,25 @@ def get_compressed_seqlens(cu_seqlens: torch.Tensor, kernel_size: int, kernel_st
 
 def last_dim_contiguous(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 else t.contiguous()
+
+
+# Head sizes the attention and decode kernels are compiled for.  Any other multiple of 8 up to the largest runs on the
+# next built size with zero columns appended to q, k and v (they add nothing to a score, and the output columns they
+# produce are zero and dropped), as the reference's kernels do inside their tiles with BLOCK_SIZE_D =
+# next_power_of_2(head_dim) and masked loads (ops/triton/topk_sparse_attention.py:866).  Here the host appends the
+# columns: one extra copy of the operands for such head sizes, none for the built ones.
+BUILT_HEAD_DIMS = (32, 64, 96, 128)
+
+
+def built_head_dim(head_dim: int) -> int:
+    assert head_dim % 8 == 0 and 0 < head_dim <= BUILT_HEAD_DIMS[-1], "head_dim must be a multiple of 8, at most %d" % BUILT_HEAD_DIMS[-1]
+    return next(d for d in BUILT_HEAD_DIMS if d >= head_dim)
+
+
+def pad_head_dim(*tensors):
+    """The tensors with their last dimension zero-padded to the built head size (unchanged when it is one)."""
+    d = tensors[0].shape[-1]
+    D = built_head_dim(d)
+    if D == d:
+        return tensors
+    return tuple(torch.nn.functional.pad(t, (0, D - d)) for t in tensors)
