@@ -28,7 +28,13 @@ HQ, HKV, D, BS = 64, 4, 128, 64
 H100_FWD_BWD_MS = 12.417 + 15.154
 # memory-side traffic per launch at the default workload (N=32768, top16), bytes: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, scaled by what the same counters read for a plain 1 GiB copy (x2.0 and x1.0); see profiles/
-MEASURED_TRAFFIC = {"topk_fwd_kernel": 15.55 * 2**30, "dq_kernel": 16.48 * 2**30, "dkdv_kernel": 18.27 * 2**30}
+MEASURED_TRAFFIC = {"topk_fwd_sweep_kernel": None, "dq_sweep_kernel": None, "dkdv_kernel": 18.27 * 2**30}
+
+
+def _paced(N):
+    """Whether the forward and the dQ pass of a sequence of N tokens run their paced schedule (pace_pays in csrc/pace.h:
+    the K/V rows of a kv-head reach 12 MiB), i.e. which kernel name a profile of the run shows."""
+    return N * D * 4 >= 12 << 20
 
 
 def _events_ms(fn, iters):
@@ -67,11 +73,24 @@ def cpu_baseline():
             if i > 0:
                 times.append(time.perf_counter() - t0)
     med = statistics.median(times)
-    return {
+    out = {
         "value": flops / med / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port", "ms": med * 1e3,
         "sample": "oracle forward, fp32, cu_seqlens=[0,512,1536,2048], 16 q / 1 kv heads, d=64, block 64, top-8 "
                   "(block 0 and own block forced), seed 0; 1 warm-up, median of 7 runs",
     }
+    if torch.cuda.is_available():
+        # the same inputs (cast to bf16) through the HIP operator, for the record beside the host figure
+        from native_sparse_attention.ops import topk_sparse_attention
+        dev = torch.device("cuda:0")
+        qg, kg, vg, ig, cg = q.bfloat16().to(dev), k.bfloat16().to(dev), v.bfloat16().to(dev), idx.to(dev), cu.to(dev)
+        with torch.no_grad():
+            for _ in range(3):
+                topk_sparse_attention(qg, kg, vg, ig, 64, cg)
+            torch.cuda.synchronize()
+            gpu_ms = _events_ms(lambda: topk_sparse_attention(qg, kg, vg, ig, 64, cg), 20)
+        out["gpu_ms_same_inputs_bf16"] = gpu_ms
+        out["gpu_over_cpu"] = med * 1e3 / gpu_ms
+    return out
 
 
 def _mfma_roofline(ops, whole_tflops):
@@ -380,8 +399,8 @@ def measure_topk(N, topk, steps, warmup, dev, per_kernel):
         small = idx.numel() * 4 + 2 * HQ * N * 4               # block ids, lse / delta
         out["kernels"] = {
             # name: (ms, algorithmic FLOPs per launch, bytes the kernel must read or write at least once)
-            "topk_fwd_kernel": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd, 2 * qb + 2 * kvb + small),              # QK^T, PV
-            "dq_kernel": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd, 4 * qb + 2 * kvb + small),                   # dS K (recomputed QK^T, dO V^T not counted)
+            "topk_fwd_sweep_kernel" if _paced(N) else "topk_fwd_kernel": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd, 2 * qb + 2 * kvb + small),   # QK^T, PV
+            "dq_sweep_kernel" if _paced(N) else "dq_kernel": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd, 4 * qb + 2 * kvb + small),            # dS K (recomputed QK^T, dO V^T not counted)
             "dkdv_kernel": (_events_ms(lambda: bwd(2), it), 2.0 * f_fwd, 2 * qb + 4 * kvb + small),       # QK^T, dO V^T, P^T dO, dS^T Q
             "reverse_index": (_events_ms(lambda: bwd(1), it) , 0.0, None),   # run alone this phase also holds the stand-alone delta pass
         }
@@ -456,7 +475,7 @@ def main():
     }
     if not args.no_sweep:
         sweep = []
-        for n in (2048, 4096, 8192, 16384, 32768, 65536):
+        for n in (2048, 4096, 8192, 16384, 32768, 65536, 131072):
             for kk in (8, 16):
                 m = r if (n, kk) == (N, topk) else measure_topk(n, kk, max(3, min(args.steps, 10)), 2, dev, per_kernel=False)
                 sweep.append({"N": n, "topk": kk, "fwd_ms": round(m["fwd_ms"], 4), "bwd_ms": round(m["bwd_ms"], 4),

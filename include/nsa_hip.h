@@ -112,6 +112,16 @@ int nsa_pool_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlen
                  int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim, int64_t kernel_size,
                  int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h, int64_t y_stride_n, int64_t y_stride_h,
                  int64_t w_stride_h, int dtype, void* stream);
+/* The same with the reference's bias step folded in: replaces the `y + bias.unsqueeze(0)` that follows the launch
+ * (weighted_pool.py:326-329 for the weighted pool, :361 for the average).  bias [H, D] in the dtype of x (NULL: none),
+ * e.g. einsum(pe, w) or mean(pe): the pooled value is rounded to the element type, then the sum, as the tensor
+ * expression does, so the result is bit-identical to nsa_pool_fwd followed by the addition.
+ */
+int nsa_pool_fwd_bias(const void* x, const void* w, const void* bias, void* y, const int32_t* cu_seqlens,
+                      const int32_t* y_cu_seqlens, int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads,
+                      int64_t head_dim, int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
+                      int64_t y_stride_n, int64_t y_stride_h, int64_t w_stride_h, int64_t bias_stride_h, int dtype,
+                      void* stream);
 /* Backward: replaces sliding_pool_dxdw_kernel (:89-179, launched at :262-292) and the dw.sum(1)
  * that follows (:297).  dx is a gather over the windows covering each token (no atomics);
  * dw (NULL iff w is NULL) is reduced over fp32 per-tile partials held in the workspace.
@@ -135,6 +145,15 @@ int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t
                             int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
                             int64_t y_stride_n, int64_t y_stride_h, int dtype, void* workspace, size_t workspace_bytes,
                             void* stream);
+/* The same with the reference's bias step folded in: replaces the `y + bias.unsqueeze(0)` after the launch
+ * (linear_compress.py:520-524).  bias [H, D] in the dtype of x (NULL: none), i.e. pe[h].flatten() @ w[h]; rounded as
+ * the tensor expression rounds (product first, then the sum).  Needs no workspace.
+ */
+int nsa_linear_compress_fwd_bias(const void* x, const void* w, const void* bias, void* y, const int32_t* cu_seqlens,
+                                 const int32_t* y_cu_seqlens, int64_t total_x, int64_t total_y, int64_t batch,
+                                 int64_t num_heads, int64_t head_dim, int64_t kernel_size, int64_t kernel_stride,
+                                 int64_t x_stride_n, int64_t x_stride_h, int64_t y_stride_n, int64_t y_stride_h,
+                                 int64_t bias_stride_h, int dtype, void* stream);
 /* Backward: replaces linear_compress_bwd_kernel and its fp32 atomic adds (:140-306, launched at
  * :449-480).  dx [total_x,H,D]; dw [H, kernel_size*D, D] contiguous, both in the dtype of x.
  * Gather formulation, no atomics: reproducible.

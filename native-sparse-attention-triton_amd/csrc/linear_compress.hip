@@ -13,6 +13,7 @@ struct LinParams {
   const int32_t* cu; const int32_t* ycu;
   int total_x, total_y, batch, H, ks, st;
   long long xsn, xsh, ysn, ysh, dysn, dysh, dxsn, dxsh;  // w, dw: [H, ks*D, D] contiguous
+  const void* bias; long long bsh;   // forward: optional [H, D] row added to every output row (null: none)
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -166,8 +167,14 @@ __global__ __launch_bounds__(512) void lin_fwd_kernel(LinParams p) {
     const f32x4 s = (*reinterpret_cast<const f32x4*>(&part[0][row][c4]) + *reinterpret_cast<const f32x4*>(&part[1][row][c4])) +
                     (*reinterpret_cast<const f32x4*>(&part[2][row][c4]) + *reinterpret_cast<const f32x4*>(&part[3][row][c4]));
     v4 o;
+    if (p.bias) {   // y + bias as 16-bit tensor arithmetic does it: the product is rounded first, the sum again
+      const v4 bv = *reinterpret_cast<const v4*>((const T*)p.bias + (long long)h * p.bsh + c4);
 #pragma unroll
-    for (int z = 0; z < 4; z++) o[z] = (T)s[z];
+      for (int z = 0; z < 4; z++) o[z] = (T)(rounded<T>(s[z]) + (float)bv[z]);
+    } else {
+#pragma unroll
+      for (int z = 0; z < 4; z++) o[z] = (T)s[z];
+    }
     st8((T*)p.y + (long long)(p.ycu[b] + n0 + row) * p.ysn + (long long)h * p.ysh + c4, o);
   }
 }
@@ -350,6 +357,7 @@ static int lin_fill(LinParams& p, const void* x, const void* w, const int32_t* c
   if ((xsn | xsh) % 8 != 0 || ((uintptr_t)x | (uintptr_t)w) % 16 != 0) return NSA_ERR_UNSUPPORTED;
   p.x = x; p.w = w; p.cu = cu; p.ycu = ycu; p.total_x = (int)total_x; p.total_y = (int)total_y; p.batch = (int)batch; p.H = (int)H;
   p.ks = (int)ks; p.st = (int)st; p.xsn = xsn; p.xsh = xsh;
+  p.bias = nullptr; p.bsh = 0;
   p.dy = nullptr; p.y = nullptr; p.dx = nullptr; p.dw = nullptr; p.ysn = p.ysh = p.dysn = p.dysh = p.dxsn = p.dxsh = 0;
   return NSA_OK;
 }
@@ -358,18 +366,28 @@ static int lin_fill(LinParams& p, const void* x, const void* w, const int32_t* c
 // library that needed one keep working.
 extern "C" size_t nsa_linear_compress_fwd_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int64_t) { return 0; }
 
+extern "C" int nsa_linear_compress_fwd_bias(const void* x, const void* w, const void* bias, void* y, const int32_t* cu_seqlens,
+                                            const int32_t* y_cu_seqlens, int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads,
+                                            int64_t head_dim, int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n,
+                                            int64_t x_stride_h, int64_t y_stride_n, int64_t y_stride_h, int64_t bias_stride_h, int dtype,
+                                            void* stream) {
+  LinParams p;
+  int rc = lin_fill(p, x, w, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, kernel_size, kernel_stride, x_stride_n, x_stride_h, dtype);
+  if (rc != NSA_OK) return rc;
+  if (total_y > 0 && (!y || (y_stride_n | y_stride_h) % 4 != 0 || (uintptr_t)y % 8 != 0)) return NSA_ERR_UNSUPPORTED;
+  if (bias && (bias_stride_h % 4 != 0 || (uintptr_t)bias % 8 != 0)) return NSA_ERR_UNSUPPORTED;
+  p.y = y; p.ysn = y_stride_n; p.ysh = y_stride_h; p.bias = bias; p.bsh = bias_stride_h;
+  return lin_dispatch(p, 0, head_dim, dtype, (hipStream_t)stream);
+}
+
 extern "C" int nsa_linear_compress_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
                                        int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
                                        int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
                                        int64_t y_stride_n, int64_t y_stride_h, int dtype, void* workspace, size_t workspace_bytes,
                                        void* stream) {
-  LinParams p;
-  int rc = lin_fill(p, x, w, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, kernel_size, kernel_stride, x_stride_n, x_stride_h, dtype);
-  if (rc != NSA_OK) return rc;
-  if (total_y > 0 && (!y || (y_stride_n | y_stride_h) % 4 != 0 || (uintptr_t)y % 8 != 0)) return NSA_ERR_UNSUPPORTED;
-  p.y = y; p.ysn = y_stride_n; p.ysh = y_stride_h;
   (void)workspace; (void)workspace_bytes;
-  return lin_dispatch(p, 0, head_dim, dtype, (hipStream_t)stream);
+  return nsa_linear_compress_fwd_bias(x, w, nullptr, y, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, head_dim, kernel_size,
+                                      kernel_stride, x_stride_n, x_stride_h, y_stride_n, y_stride_h, 0, dtype, stream);
 }
 
 extern "C" int nsa_linear_compress_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, const int32_t* cu_seqlens,

@@ -10,7 +10,23 @@ struct PoolParams {
   const void* x; const void* w; const void* y; const int32_t* cu; const int32_t* ycu;
   int total_x, total_y, batch, H, ks, st;
   long long xsn, xsh, ysn, ysh, wsh;
+  const void* bias; long long bsh;   // optional [H, D] row added to every output row (null: none)
 };
+
+// out = y + bias as 16-bit tensor arithmetic does it: the pooled value is rounded to the element type first, the sum again
+template <typename T, typename V8>
+__device__ __forceinline__ V8 pooled_row_piece(const float (&acc)[8], const void* bias, long long bsh, int h, int c) {
+  V8 out;
+  if (bias) {
+    const V8 b = ld16<V8>((const T*)bias + (long long)h * bsh + 8 * c);
+#pragma unroll
+    for (int j = 0; j < 8; j++) out[j] = (T)(rounded<T>(acc[j]) + (float)b[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; j++) out[j] = (T)acc[j];
+  }
+  return out;
+}
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) void pool_fwd_kernel(PoolParams p, T* __restrict__ y) {
@@ -47,9 +63,7 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(PoolParams p, T* __restri
 #pragma unroll
     for (int j = 0; j < 8; j++) acc[j] = __builtin_fmaf(wk, (float)xv[j], acc[j]);
   }
-  v8 out;
-#pragma unroll
-  for (int j = 0; j < 8; j++) out[j] = (T)acc[j];
+  const v8 out = pooled_row_piece<T, v8>(acc, p.bias, p.bsh, h, c);
   st16(y + (long long)n * p.ysn + (long long)h * p.ysh + 8 * c, out);
 }
 
@@ -101,9 +115,7 @@ __global__ __launch_bounds__(256) void pool_fwd_split_kernel(PoolParams p, T* __
       for (int j = 0; j < 8; j++) acc[j] += part[s2 - 1][pl][j];
   }
   if (!live) return;
-  v8 out;
-#pragma unroll
-  for (int j = 0; j < 8; j++) out[j] = (T)acc[j];
+  const v8 out = pooled_row_piece<T, v8>(acc, p.bias, p.bsh, h, c);
   st16(y + (long long)n * p.ysn + (long long)h * p.ysh + 8 * c, out);
 }
 
@@ -243,23 +255,33 @@ static int fill_params(PoolParams& p, const void* x, const void* w, const int32_
   if ((xsn | xsh) % 8 != 0 || (uintptr_t)x % 16 != 0) return NSA_ERR_UNSUPPORTED;
   p.x = x; p.w = w; p.cu = cu; p.ycu = ycu; p.total_x = (int)total_x; p.total_y = (int)total_y; p.batch = (int)batch;
   p.H = (int)H; p.ks = (int)ks; p.st = (int)st; p.xsn = xsn; p.xsh = xsh; p.wsh = wsh; p.y = nullptr; p.ysn = p.ysh = 0;
+  p.bias = nullptr; p.bsh = 0;
   return NSA_OK;
+}
+
+extern "C" int nsa_pool_fwd_bias(const void* x, const void* w, const void* bias, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
+                                 int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
+                                 int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
+                                 int64_t y_stride_n, int64_t y_stride_h, int64_t w_stride_h, int64_t bias_stride_h, int dtype, void* stream) {
+  PoolParams p;
+  int rc = fill_params(p, x, w, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, kernel_size, kernel_stride, x_stride_n, x_stride_h, w_stride_h);
+  if (rc != NSA_OK) return rc;
+  if (total_y > 0 && (!y || (y_stride_n | y_stride_h) % 8 != 0 || (uintptr_t)y % 16 != 0)) return NSA_ERR_UNSUPPORTED;
+  if (bias && (bias_stride_h % 8 != 0 || (uintptr_t)bias % 16 != 0)) return NSA_ERR_UNSUPPORTED;
+  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
+  p.ysn = y_stride_n; p.ysh = y_stride_h; p.bias = bias; p.bsh = bias_stride_h;
+  hipStream_t s = (hipStream_t)stream;
+#define CALL(T, D) pool_fwd_t<T, D>(p, y, s)
+  POOL_DISPATCH(CALL)
+#undef CALL
 }
 
 extern "C" int nsa_pool_fwd(const void* x, const void* w, void* y, const int32_t* cu_seqlens, const int32_t* y_cu_seqlens,
                             int64_t total_x, int64_t total_y, int64_t batch, int64_t num_heads, int64_t head_dim,
                             int64_t kernel_size, int64_t kernel_stride, int64_t x_stride_n, int64_t x_stride_h,
                             int64_t y_stride_n, int64_t y_stride_h, int64_t w_stride_h, int dtype, void* stream) {
-  PoolParams p;
-  int rc = fill_params(p, x, w, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, kernel_size, kernel_stride, x_stride_n, x_stride_h, w_stride_h);
-  if (rc != NSA_OK) return rc;
-  if (total_y > 0 && (!y || (y_stride_n | y_stride_h) % 8 != 0 || (uintptr_t)y % 16 != 0)) return NSA_ERR_UNSUPPORTED;
-  if (dtype != NSA_BF16 && dtype != NSA_FP16) return NSA_ERR_UNSUPPORTED;
-  p.ysn = y_stride_n; p.ysh = y_stride_h;
-  hipStream_t s = (hipStream_t)stream;
-#define CALL(T, D) pool_fwd_t<T, D>(p, y, s)
-  POOL_DISPATCH(CALL)
-#undef CALL
+  return nsa_pool_fwd_bias(x, w, nullptr, y, cu_seqlens, y_cu_seqlens, total_x, total_y, batch, num_heads, head_dim, kernel_size,
+                           kernel_stride, x_stride_n, x_stride_h, y_stride_n, y_stride_h, w_stride_h, 0, dtype, stream);
 }
 
 extern "C" size_t nsa_pool_bwd_workspace_bytes(int64_t total_y, int64_t num_heads, int64_t kernel_size) {

@@ -24,6 +24,7 @@ _SIGNATURES = {
     "nsa_topk_reverse_index_segments": (I, [I] * 4),
     "nsa_topk_attn_bwd": (c_int, [P] * 11 + [I] * 7 + [P, F, c_int, P, Z, P, P, c_int, P]),
     "nsa_pool_fwd": (c_int, [P] * 5 + [I] * 12 + [c_int, P]),
+    "nsa_pool_fwd_bias": (c_int, [P] * 6 + [I] * 13 + [c_int, P]),
     "nsa_pool_bwd_workspace_bytes": (Z, [I] * 3),
     "nsa_pool_bwd": (c_int, [P] * 7 + [I] * 15 + [c_int, P, Z, P]),
     "nsa_dense_decode_workspace_bytes": (Z, [I] * 5),
@@ -39,6 +40,7 @@ _SIGNATURES = {
     "nsa_cmp_attn_bwd": (c_int, [P] * 11 + [I] * 8 + [P, F, c_int, P, Z, P]),
     "nsa_linear_compress_fwd_workspace_bytes": (Z, [I] * 5),
     "nsa_linear_compress_fwd": (c_int, [P] * 5 + [I] * 11 + [c_int, P, Z, P]),
+    "nsa_linear_compress_fwd_bias": (c_int, [P] * 6 + [I] * 12 + [c_int, P]),
     "nsa_linear_compress_bwd": (c_int, [P] * 7 + [I] * 13 + [c_int, P]),
     "nsa_window_attn_fwd": (c_int, [P] * 6 + [I] * 6 + [P, F, c_int, P]),
     "nsa_cache_fill": (c_int, [P] * 7 + [I] * 10 + [P]),

@@ -26,6 +26,32 @@ def get_compressed_seqlens(cu_seqlens: torch.Tensor, kernel_size: int, kernel_st
     return y_seqlens, y_cu_seqlens
 
 
+# Compressed lengths of the cu_seqlens tensors seen last: K and V of a layer (and every layer of a model) compress with the
+# same cu_seqlens object, and each fresh computation costs a launch plus, for the output shape, a device read.  An entry
+# is valid while the very same tensor object is alive and has not been written to (its version counter is unchanged).
+_SEQLEN_CACHE = {}
+
+
+def compressed_seqlens_cached(cu_seqlens: torch.Tensor, kernel_size: int, kernel_stride: int, need_total: bool):
+    """(y_cu_seqlens, total or None): as get_compressed_seqlens, remembered per cu_seqlens object; total = the sum of the
+    compressed lengths as a host integer (one device read, the first time it is asked for)."""
+    import weakref
+
+    key = (id(cu_seqlens), kernel_size, kernel_stride)
+    hit = _SEQLEN_CACHE.get(key)
+    if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
+        entry = hit
+    else:
+        if len(_SEQLEN_CACHE) >= 32:
+            for k_ in [k_ for k_, e in _SEQLEN_CACHE.items() if e[0]() is None] or list(_SEQLEN_CACHE)[:16]:
+                del _SEQLEN_CACHE[k_]
+        entry = [weakref.ref(cu_seqlens), cu_seqlens._version, get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)[1], None]
+        _SEQLEN_CACHE[key] = entry
+    if need_total and entry[3] is None:
+        entry[3] = int(entry[2][-1])
+    return entry[2], entry[3]
+
+
 def last_dim_contiguous(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 else t.contiguous()
 

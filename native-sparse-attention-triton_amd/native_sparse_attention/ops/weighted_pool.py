@@ -5,12 +5,12 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from .utils import get_compressed_seqlens, last_dim_contiguous
+from .utils import compressed_seqlens_cached, last_dim_contiguous
 
 
 class SlidingWindowWeightedPool(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w, cu_seqlens, kernel_size, kernel_stride, known_total=None, known_y_cu=None):
+    def forward(ctx, x, w, cu_seqlens, kernel_size, kernel_stride, known_total=None, known_y_cu=None, bias=None):
         assert x.dtype == torch.float16 or x.dtype == torch.bfloat16
         if w is not None:
             assert x.dtype == w.dtype
@@ -23,19 +23,28 @@ class SlidingWindowWeightedPool(torch.autograd.Function):
         assert kernel_size % kernel_stride == 0
         assert kernel_size in {16, 32, 64, 128}
         x = last_dim_contiguous(x)
-        y_cu_seqlens = known_y_cu if known_y_cu is not None else get_compressed_seqlens(cu_seqlens, kernel_size, kernel_stride)[1]
-        # output shape: the one host synchronisation the reference has too, unless the caller knows the total
-        total_y = int(y_cu_seqlens[-1]) if known_total is None else int(known_total)
+        # compressed lengths and the output shape: a launch and the one host synchronisation the reference has too,
+        # unless the caller passes them or this cu_seqlens tensor has been through here before
+        if known_y_cu is not None and known_total is not None:
+            y_cu_seqlens, total_y = known_y_cu, int(known_total)
+        else:
+            y_cu_seqlens, total_y = compressed_seqlens_cached(cu_seqlens, kernel_size, kernel_stride, known_total is None)
+            y_cu_seqlens = known_y_cu if known_y_cu is not None else y_cu_seqlens
+            total_y = int(known_total) if known_total is not None else total_y
+        if bias is not None:
+            assert bias.shape == (num_heads, head_dim) and bias.dtype == x.dtype
+            bias = bias.contiguous()
         y = torch.empty(total_y, num_heads, head_dim, dtype=x.dtype, device=x.device)
         lib = _lib.load()
-        rc = lib.nsa_pool_fwd(
-            x.data_ptr(), w.data_ptr() if w is not None else None, y.data_ptr(), cu_seqlens.data_ptr(),
-            y_cu_seqlens.data_ptr(), total_len, total_y, batch, num_heads, head_dim, kernel_size, kernel_stride,
+        rc = lib.nsa_pool_fwd_bias(
+            x.data_ptr(), w.data_ptr() if w is not None else None, bias.data_ptr() if bias is not None else None, y.data_ptr(),
+            cu_seqlens.data_ptr(), y_cu_seqlens.data_ptr(), total_len, total_y, batch, num_heads, head_dim, kernel_size, kernel_stride,
             x.stride(0), x.stride(1), y.stride(0), y.stride(1), w.stride(0) if w is not None else 0,
-            _lib.dtype_code(x), _lib.stream_ptr(x))
+            bias.stride(0) if bias is not None else 0, _lib.dtype_code(x), _lib.stream_ptr(x))
         _lib.check(rc, "nsa_pool_fwd")
         ctx.save_for_backward(x, w, cu_seqlens, y_cu_seqlens)
         ctx.kernel_size, ctx.kernel_stride, ctx.total_y = kernel_size, kernel_stride, total_y
+        ctx.has_bias = bias is not None
         ctx.mark_non_differentiable(y_cu_seqlens)
         return y, y_cu_seqlens
 
@@ -57,7 +66,9 @@ class SlidingWindowWeightedPool(torch.autograd.Function):
             w.stride(0) if w is not None else 0, dw.stride(0) if w is not None else 0,
             _lib.dtype_code(x), ws.data_ptr(), ws.numel(), _lib.stream_ptr(x))
         _lib.check(rc, "nsa_pool_bwd")
-        return dx, dw, None, None, None, None, None
+        # the bias row was added to every output row
+        dbias = dy.sum(0) if ctx.has_bias else None
+        return dx, dw, None, None, None, None, None, dbias
 
 
 def weightedpool_compress(
@@ -79,12 +90,11 @@ def weightedpool_compress(
     host; the output is then allocated without reading y_cu_seqlens back.  known_y_cu (likewise): the output's
     cu_seqlens when the caller already holds them (a decode step compresses one full window per sequence).
     """
-    y, y_cu_seqlens = SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu)
+    bias = None
     if pe is not None:
         assert pe.dtype == x.dtype and pe.device == x.device
-        bias = torch.einsum("hkd,hk->hd", pe, w)
-        y = y + bias.unsqueeze(0)
-    return y, y_cu_seqlens
+        bias = torch.einsum("hkd,hk->hd", pe, w)   # added to every output row by the kernel
+    return SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu, bias)
 
 
 def avgpool_compress(
@@ -100,8 +110,8 @@ def avgpool_compress(
     """Average sliding-window pooling; ``w`` must be None.  Bias = mean_k pe[h,k,:].  known_total / known_y_cu as in
     weightedpool_compress."""
     assert w is None, "don't need additional weight for avgpool"
-    y, y_cu_seqlens = SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu)
+    bias = None
     if pe is not None:
         assert pe.dtype == x.dtype and pe.device == x.device
-        y = y + torch.mean(pe, dim=1).unsqueeze(0)
-    return y, y_cu_seqlens
+        bias = torch.mean(pe, dim=1)   # added to every output row by the kernel
+    return SlidingWindowWeightedPool.apply(x, w, cu_seqlens, kernel_size, kernel_stride, known_total, known_y_cu, bias)
