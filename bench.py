@@ -31,10 +31,10 @@ H100_FWD_BWD_MS = 12.417 + 15.154
 MEASURED_TRAFFIC = {"topk_fwd_sweep_kernel": None, "dq_sweep_kernel": None, "dkdv_kernel": 18.27 * 2**30}
 
 
-def _paced(N):
+def _paced(N, topk):
     """Whether the forward and the dQ pass of a sequence of N tokens run their paced schedule (pace_pays in csrc/pace.h:
-    the K/V rows of a kv-head reach 12 MiB), i.e. which kernel name a profile of the run shows."""
-    return N * D * 4 >= 12 << 20
+    at least 8 blocks per token and K/V rows of a kv-head that reach 12 MiB), i.e. which kernel name a profile shows."""
+    return topk >= 8 and N * D * 4 >= 12 << 20
 
 
 def _events_ms(fn, iters):
@@ -399,8 +399,8 @@ def measure_topk(N, topk, steps, warmup, dev, per_kernel):
         small = idx.numel() * 4 + 2 * HQ * N * 4               # block ids, lse / delta
         out["kernels"] = {
             # name: (ms, algorithmic FLOPs per launch, bytes the kernel must read or write at least once)
-            "topk_fwd_sweep_kernel" if _paced(N) else "topk_fwd_kernel": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd, 2 * qb + 2 * kvb + small),   # QK^T, PV
-            "dq_sweep_kernel" if _paced(N) else "dq_kernel": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd, 4 * qb + 2 * kvb + small),            # dS K (recomputed QK^T, dO V^T not counted)
+            "topk_fwd_sweep_kernel" if _paced(N, topk) else "topk_fwd_kernel": (_events_ms(lambda: fwd(2), it), 1.0 * f_fwd, 2 * qb + 2 * kvb + small),   # QK^T, PV
+            "dq_sweep_kernel" if _paced(N, topk) else "dq_kernel": (_events_ms(lambda: bwd(4), it), 0.5 * f_fwd, 4 * qb + 2 * kvb + small),            # dS K (recomputed QK^T, dO V^T not counted)
             "dkdv_kernel": (_events_ms(lambda: bwd(2), it), 2.0 * f_fwd, 2 * qb + 4 * kvb + small),       # QK^T, dO V^T, P^T dO, dS^T Q
             "reverse_index": (_events_ms(lambda: bwd(1), it) , 0.0, None),   # run alone this phase also holds the stand-alone delta pass
         }

@@ -45,7 +45,7 @@ int nsa_version(void);
  * nsa_topk_attn_fwd_workspace_bytes().
  * phases: NSA_FWD_PHASE_ALL, or a subset when the caller re-uses the workspace of a previous
  * call with the same K and V (profiling a single kernel).
- * Schedule: when the K/V rows of one kv-head reach 12 MiB (24 K tokens of 128 columns) the attend pass runs
+ * Schedule: when topk >= 8 and the K/V rows of one kv-head reach 12 MiB (24 K tokens of 128 columns) the attend pass runs
  * as persistent waves whose key positions are kept within a window of each other, so that an XCD's L2 serves
  * most of the block fetches; below that, one wave per token in launch order.  Both give bit-identical
  * results.  Or-ing NSA_FWD_SCHEDULE_PLAIN or NSA_FWD_SCHEDULE_PACED into phases forces one of them.

@@ -75,12 +75,14 @@ static __global__ __launch_bounds__(1024) void pace_prepare_kernel(int32_t* __re
   }
 }
 
-// Which launches are paced, and how.  Measured on single sequences of 64 q / 4 kv heads, 128 columns, top-16 (forward /
-// dQ pass, ms, plain -> paced): 16 K tokens 1.35 -> 1.26..1.47 / -, 32 K 2.9 -> 2.65 / 3.1 -> 3.0, 64 K 9.1 -> 5.7 /
-// 9.2 -> 6.5, 128 K 23.7 -> 13.6: pacing pays once the K/V of a kv-head is several times the 4 MiB of an L2.
+// Which launches are paced, and how.  Measured on single sequences of 64 q / 4 kv heads, 128 columns (forward, ms,
+// plain -> paced): top-16 at 16 K tokens 1.31 -> 1.45, 32 K 2.9 -> 2.65, 64 K 9.1 -> 5.7, 128 K 23.7 -> 13.6; top-8 at
+// 16 K 0.78 -> 0.78, 32 K 1.63 -> 1.58, 64 K 4.1 -> 3.6, 128 K 10.2 -> 9.1; top-4 (one random block per token) 32 K
+// 0.89 -> 1.02, 64 K 1.9 -> 2.4.  The dQ pass: top-16 at 32 K 3.1 -> 3.0, 64 K 9.2 -> 6.5; top-8 unchanged.  Pacing
+// pays once the K/V of a kv-head is several times the 4 MiB of an L2 and a token fetches enough blocks that miss it.
 // Window: best at 160..240 positions of 32 KiB (K and V rows of 64 keys); below, waves wait for each other (a wave's
-// next block is on average topk-th of its prefix away), above, the L2 loses the window.
-static inline bool pace_pays(long long total_len, int head_dim) { return total_len * head_dim * 4 >= (12ll << 20); }
+// next block is on average a topk-th of its prefix away), above, the L2 loses the window.
+static inline bool pace_pays(long long total_len, int head_dim, int topk) { return topk >= 8 && total_len * head_dim * 4 >= (12ll << 20); }
 static inline int pace_window_units(int head_dim) { return (int)((25ll << 18) / (64 * head_dim * 4)); }  // 6.25 MiB
 static inline int pace_slots() {
   int dev = 0, cus = 256;

@@ -622,7 +622,7 @@ static int run_bwd(const BwdArgs& a) {
     p.ish = a.ish; p.isn = a.isn; p.isk = a.isk; p.dqsn = a.dqsn; p.dqsh = a.dqsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale;
     p.sched = nsa_xcd_schedule(a.T, a.B, GT * (int)a.Hkv, (int)a.D, 8.0);
-    const bool paced = (a.phases & NSA_BWD_SCHEDULE_PACED) || (!(a.phases & NSA_BWD_SCHEDULE_PLAIN) && pace_pays(a.T, (int)a.D));
+    const bool paced = (a.phases & NSA_BWD_SCHEDULE_PACED) || (!(a.phases & NSA_BWD_SCHEDULE_PLAIN) && pace_pays(a.T, (int)a.D, (int)a.topk));
     if (paced) {
       PaceParams pace;
       pace.table = (int32_t*)(ws + L.pace);

@@ -455,7 +455,7 @@ extern "C" int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, co
   // fixed part of a sweep's cost in the XCD schedule, in 64-key positions: fitted to the per-XCD times of paced
   // launches at 32 K .. 128 K tokens (1300 balances 32 K, 2500 the longer ones)
   c.fixed_units = 2000;
-  const bool paced = (phases & NSA_FWD_SCHEDULE_PACED) || (!(phases & NSA_FWD_SCHEDULE_PLAIN) && pace_pays(total_len, (int)head_dim));
+  const bool paced = (phases & NSA_FWD_SCHEDULE_PACED) || (!(phases & NSA_FWD_SCHEDULE_PLAIN) && pace_pays(total_len, (int)head_dim, (int)topk));
   if (paced) pace_fill_params(c.pace, total_len, pace_slots(), c.tokens_per_wave, pace_window_units((int)head_dim));
   if (dtype == NSA_BF16) return dispatch_d<__bf16>((int)head_dim, (int)block_size, c);
   if (dtype == NSA_FP16) return dispatch_d<_Float16>((int)head_dim, (int)block_size, c);
