@@ -185,6 +185,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // TPW = 1 is launched: with two tokens per wave (a block that both select is fetched once, half as many sweeps
 // stream the prefix) the state no longer fits 256 registers beside the 128 of a block in flight, and the spills cost
 // more than the sharing saves (forward at 32 K / 64 K / 128 K tokens: 2.84 / 6.14 / 14.9 ms against 2.75 / 5.74 / 13.9).
+// Also measured and dropped: the same kernel with a wave's fetches software-pipelined over its blocks (the next slice's
+// K fragments requested right after the score MFMAs, its V fragments after the P V MFMAs, into the registers just
+// consumed): 2.60 against 2.59 ms at 32 K tokens, 5.77 / 5.76 at 64 K - the launch is bound by what the L2 hands to the
+// L1s (63 GiB per launch at 64 B per clock and compute unit would take 1.75 ms), not by a wave's own exposed latency.
 template <typename T, int D> struct FwdToken : SweepToken {
   typename Elem<T>::v8 qf[D / 32];
   f32x4 acc[D / 16];
