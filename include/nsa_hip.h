@@ -28,6 +28,7 @@ extern "C" {
 #define NSA_ERR_UNSUPPORTED (-2)  /* head_dim / block_size / dtype outside the built set */
 #define NSA_ERR_WORKSPACE (-3)    /* workspace_bytes smaller than nsa_*_workspace_bytes  */
 #define NSA_ERR_LAUNCH (-4)       /* hipGetLastError() after the launch was not success  */
+#define NSA_ERR_NOT_READY (-5)    /* nsa_topk_decode_static: first call on this device made while the stream records a graph */
 
 #define NSA_BF16 0
 #define NSA_FP16 1

@@ -536,11 +536,16 @@ static constexpr int STATIC_MAX_DEVICES = 64;
 static void* scratch_addr[STATIC_MAX_DEVICES];   // per device, filled on the first call with that device current
 static std::mutex scratch_mutex;
 
-static int static_scratch(void** out) {
+static int static_scratch(void** out, hipStream_t stream) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return NSA_ERR_LAUNCH;
   std::lock_guard<std::mutex> hold(scratch_mutex);
   if (!scratch_addr[dev]) {
+    // the address lookup is not a stream operation: made while the caller's stream records a graph it would fail
+    // or break the recording, so that case is refused with a code of its own before anything is attempted
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) return NSA_ERR_LAUNCH;
+    if (capturing != hipStreamCaptureStatusNone) return NSA_ERR_NOT_READY;
     void* ptr = nullptr;
     if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return NSA_ERR_LAUNCH;
     scratch_addr[dev] = ptr;
@@ -559,7 +564,7 @@ extern "C" int nsa_topk_decode_static(const void* q, const void* k, const void* 
   if (nsa_topk_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, topk, block_size) > STATIC_SCRATCH_BYTES)
     return NSA_ERR_WORKSPACE;
   void* ws = nullptr;
-  const int rc = static_scratch(&ws);
+  const int rc = static_scratch(&ws, (hipStream_t)stream);
   if (rc != NSA_OK) return rc;
   // the partial kernel writes every (m, l, O) slot the merge kernel reads, so nothing left behind by an
   // earlier call needs clearing

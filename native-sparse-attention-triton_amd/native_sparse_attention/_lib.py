@@ -13,7 +13,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 _lib = None
 
 NSA_BF16, NSA_FP16 = 0, 1
-_ERR = {-1: "bad argument", -2: "unsupported shape/dtype/alignment", -3: "workspace too small", -4: "kernel launch failed"}
+_ERR = {-1: "bad argument", -2: "unsupported shape/dtype/alignment", -3: "workspace too small", -4: "kernel launch failed",
+        -5: "first call on this device made under graph capture (call once outside a capture first)"}
 
 P, I, F, Z = c_void_p, c_int64, c_float, c_size_t
 _SIGNATURES = {

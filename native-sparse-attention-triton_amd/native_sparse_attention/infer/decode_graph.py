@@ -22,8 +22,9 @@ class NSADecodeGraph:
     been filled by a prefill of the same batch before the first `step`; a later prefill of another batch of the same
     size into the same cache can reuse the object.  Replays run on the stream that is current when `step` is called.
 
-    A recorded step cannot look at lengths on the host, so the object counts its replays since the last prefill and
-    raises once the longest sequence would outgrow the cache (`max_prompt_len + steps > cache.max_length`).  The
+    A recorded step cannot look at lengths on the host, so every replay is counted on the cache (`NSACache.count_decode_step`,
+    which eager decode steps and other graphs recorded on the same cache go through as well) and raises once the longest
+    sequence would outgrow the cache (`max_prompt_len + decode_steps > cache.max_length`).  The
     kernels themselves never write past a slab either: a sequence that has filled its rows is left as it is
     (no token stored, length not advanced), which keeps memory safe but would make later outputs meaningless.
     """
@@ -36,7 +37,6 @@ class NSADecodeGraph:
         batch = cu_seqlens.shape[0] - 1
         dev, dt = cache.sparse_kv_cache.device, cache.dtype
         self.cache = cache
-        self._steps, self._prefill_serial = 0, cache.prefill_serial
         self.query = torch.zeros(batch, num_q_heads, cache.head_dim, dtype=dt, device=dev)
         self.key = torch.zeros(batch, cache.num_kv_heads, cache.head_dim, dtype=dt, device=dev)
         self.value = torch.zeros_like(self.key)
@@ -51,12 +51,8 @@ class NSADecodeGraph:
                                  local_blocks, window_size)
 
     def _count_step(self):
-        if self._prefill_serial != self.cache.prefill_serial:   # a new batch has been prefilled into the cache
-            self._steps, self._prefill_serial = 0, self.cache.prefill_serial
-        self._steps += 1
-        if self.cache.max_prompt_len + self._steps > self.cache.max_length:
-            raise RuntimeError("decode step %d of a %d-token prompt does not fit the cache (max_length %d)"
-                               % (self._steps, self.cache.max_prompt_len, self.cache.max_length))
+        # the cache keeps one count for eager steps, this graph's replays and any other graph recorded on it
+        self.cache.count_decode_step()
 
     @torch.no_grad()
     def step(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, gate_value: torch.Tensor) -> torch.Tensor:

@@ -74,7 +74,8 @@ class NSACache:
         self.dtype, self.device = dtype, device
         self.max_comp_length = (max_length - kernel_size) // kernel_stride + 1
         self.max_prompt_len = 0  # host copy of the longest prompt of the current batch (set at prefill)
-        self.prefill_serial = 0  # counts prefills: a recorded decode step restarts its step count when this changes
+        self.prefill_serial = 0  # counts prefills
+        self.decode_steps = 0    # tokens appended per sequence since the prefill, whoever ran the steps (host copy)
         self._staging_cu = None
         self._staging_out_cu = None
         self.static_shapes = False  # decode steps use the full slab extents instead of the current length bound
@@ -95,6 +96,16 @@ class NSACache:
         for t in (self.sparse_kv_len, self.compress_kv_len, self.before_compress_kv_len, self.sliding_kv_len):
             t.zero_()
         self.max_prompt_len = 0
+        self.decode_steps = 0
+
+    def count_decode_step(self):
+        """Called once per decode step that appends a token to every sequence - by the eager path and by replays of a
+        recorded step alike, so that steps of either kind on one cache are counted together.  Raises when the longest
+        sequence would outgrow its slab (the kernels would then silently stop storing tokens)."""
+        if self.max_prompt_len + self.decode_steps + 1 > self.max_length:
+            raise RuntimeError("decode step %d of a %d-token prompt does not fit the cache (max_length %d)"
+                               % (self.decode_steps + 1, self.max_prompt_len, self.max_length))
+        self.decode_steps += 1
 
     def staging_cu_seqlens(self, batch: int) -> torch.Tensor:
         """cu_seqlens of the staging slab seen as a varlen batch: every sequence contributes kernel_size rows."""
@@ -156,6 +167,8 @@ class NSACache:
         for w in (weight_k, weight_v):
             assert w is None or (w.dtype == self.dtype and w.is_contiguous() and w.shape == (self.num_kv_heads, self.kernel_size))
         assert bias_k is None or (bias_k.dtype == self.dtype and bias_k.is_contiguous() and bias_k.shape == (self.num_kv_heads, self.head_dim))
+        if not torch.cuda.is_current_stream_capturing():   # a capture records the launch without running it
+            self.count_decode_step()
         out = torch.empty_like(query, memory_format=torch.contiguous_format)
         strides = _lib.host_i64([query.stride(0), query.stride(1), key.stride(0), key.stride(1), value.stride(0), value.stride(1),
                                  out.stride(0), out.stride(1)])
@@ -179,6 +192,7 @@ class NSACache:
             seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
             self.max_prompt_len = int(seqlens.max())  # the one host read of a prefill
             self.prefill_serial += 1
+            self.decode_steps = 0
             assert self.max_prompt_len <= self.max_length
             _, comp_cu = get_compressed_seqlens(cu_seqlens, self.kernel_size, self.kernel_stride)
             self._fill(self.compress_kv_cache, self.compress_kv_len, compress_key, compress_value, comp_cu,
@@ -190,6 +204,8 @@ class NSACache:
             self._fill(self.sliding_kv_cache, self.sliding_kv_len, sliding_key, sliding_value, cu_seqlens, start, cu_seqlens[1:].contiguous())
         else:
             assert self.static_shapes or self.max_seqlen(step) <= self.max_length, "cache slab too short for this decode step"
+            if not torch.cuda.is_current_stream_capturing():
+                self.count_decode_step()
             toks = [last_dim_contiguous(t) for t in (compress_key, compress_value, sparse_key, sparse_value, sliding_key, sliding_value)]
             assert all(t.shape[0] == batch and t.dtype == self.dtype for t in toks)
             ptrs = (ctypes.c_void_p * 6)(*[t.data_ptr() for t in toks])

@@ -107,3 +107,29 @@ def test_negative_softmax_scale(device):
     assert_close(o, want, "o")
     qb = torch.cat([torch.arange(L, device=device) for L in (300, 200)]) // 64
     assert_ids_match(idx, want_idx, bscore, qb, "topk_idx", min_overlap=0.9)
+
+
+@pytest.mark.parametrize("scale", [-0.2, 0.0])
+def test_any_finite_scale_forward_and_backward(device, scale):
+    """Every entry point of the compressed-attention family takes any finite softmax scale: forward, selection and both
+    backward kernels at a negative and at a zero scale (all probabilities equal among the visible keys)."""
+    lens, Hq, Hkv, d, ks, st, bs, topk = [300, 700], 8, 2, 64, 32, 16, 64, 4
+    q, ck, cv, cu, cuk = _inputs(lens, Hq, Hkv, d, ks, st, torch.bfloat16, device, seed=5)
+    q = (q.float() * 0.3).bfloat16()
+    q1, k1, v1 = (x.clone().requires_grad_() for x in (q, ck, cv))
+    o, idx = compressed_attention(q1, k1, v1, ks, st, bs, topk, cu, cuk, max(lens), None, scale)
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, ck, cv))
+    want, want_idx, bscore = oracle.compressed_attention(qf, kf, vf, ks, st, bs, topk, cu, cuk, max(lens), None, scale, return_scores=True)
+    assert_close(o, want, "o")
+    g = torch.Generator(device=device).manual_seed(8)
+    do = torch.randn(o.shape, generator=g, device=device).to(o.dtype)
+    o.backward(do)
+    want.backward(do.float())
+    for name, a, b in (("dq", q1.grad, qf.grad), ("dk", k1.grad, kf.grad), ("dv", v1.grad, vf.grad)):
+        assert_close(a, b, name, rel_to=True)
+    qb = torch.cat([torch.arange(L, device=device) for L in lens]) // bs
+    # at scale 0 every block score ties with its neighbours: only the shape and the forced blocks are fixed
+    if scale != 0.0:
+        assert_ids_match(idx, want_idx, bscore, qb, "topk_idx", min_overlap=0.9)
+    else:
+        assert idx.shape == want_idx.shape and (idx[..., 0] == 0).all() and (idx == qb[None, :, None]).any(-1).all()

@@ -213,8 +213,8 @@ def test_single_launch_prepare_equals_separate_operators(device, weighted, with_
 
 
 def test_graphed_decode_refuses_to_outgrow_the_cache(device):
-    """A recorded step cannot check lengths on the host: the graph object counts its replays and raises before the
-    longest sequence would need a row the cache does not have; a new prefill restarts the count."""
+    """A recorded step cannot check lengths on the host: the cache counts the decode steps run on it (replays and eager
+    steps alike) and raises before the longest sequence would need a row it does not have; a new prefill restarts the count."""
     from native_sparse_attention.infer import NSADecodeGraph
     from native_sparse_attention.module import RopeConfig, RotaryEmbedding
     Hq, Hkv, d, ks, st, bs, topk, W = 16, 2, 128, 32, 16, 64, 4, 64
@@ -242,3 +242,12 @@ def test_graphed_decode_refuses_to_outgrow_the_cache(device):
     prefill()
     graph.step(*tok())                                 # the count restarted with the new prompt
     assert int(cache.sparse_kv_len[0]) == 71
+    # eager steps and replays on one cache are counted together: one replay above, two eager steps here, then neither fits
+    for step in (2, 3):
+        nsa_infer(cu, step, *tok(), rope, cache, *tail)
+    assert int(cache.sparse_kv_len[0]) == 73 and cache.decode_steps == 3
+    with pytest.raises(RuntimeError):
+        graph.step(*tok())
+    with pytest.raises((RuntimeError, AssertionError)):
+        nsa_infer(cu, 4, *tok(), rope, cache, *tail)
+    assert int(cache.sparse_kv_len[0]) == 73

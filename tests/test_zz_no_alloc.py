@@ -46,6 +46,39 @@ def test_static_scratch_decode_equals_workspace_decode(device):
         assert o.float().abs().max() > 0
 
 
+def test_static_scratch_decode_allocates_nothing_and_replays_from_a_graph(device):
+    q, k, v, idx, lens = _case(4, 2048, 32, 2, 128, 64, 8, torch.bfloat16, device, seed=6)
+    rc, want = _static(q, k, v, idx, 64, lens)          # first use on this device happens outside any capture
+    assert rc == 0
+    torch.cuda.synchronize()
+    o = torch.empty_like(q)
+    strides = _strides(q, k, v, o, idx)
+    lib = _lib.load()
+    call = lambda: lib.nsa_topk_decode_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), idx.data_ptr(), lens.data_ptr(), o.data_ptr(),
+                                              4, 32, 2, 128, 2048, 8, 64, strides, 128 ** -0.5, _lib.dtype_code(q), _lib.stream_ptr(q))
+    # neither the caching allocator nor the driver hands out memory for a call
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    assert call() == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.equal(o, want)
+    # recorded into a graph and replayed, with eager work and synchronisations between the replays
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = call()
+    assert rc == 0
+    for r in range(3):
+        o.zero_()
+        q.mul_(-1)                                       # other inputs each time: the graph reads the buffers, not a snapshot
+        graph.replay()
+        torch.cuda.synchronize()
+        want = topk_sparse_attention_decode(q, k, v, idx, 64, lens)
+        torch.cuda.synchronize()
+        assert torch.equal(o, want), r
+
+
 def test_static_scratch_decode_rejects_sizes_beyond_its_array(device):
     lib = _lib.load()
     B, Hq, Hkv, d, topk = 64, 64, 4, 128, 64
