@@ -164,10 +164,11 @@ def test_reverse_index_bit_exact_and_deterministic(device, lens, Hkv, bs, topk):
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
-def test_forward_backward_replayed_from_a_hip_graph(device):
+@pytest.mark.parametrize("schedule", [8, 16])   # NSA_*_SCHEDULE_PLAIN / _PACED: one wave per token / persistent paced waves
+def test_forward_backward_replayed_from_a_hip_graph(device, schedule):
     """Forward + backward recorded once into a HIP graph (nothing in them allocates, synchronises or clears memory with
-    a memset) and replayed on fresh inputs, with eager work and synchronisation between the replays: every replay
-    must equal the eager result bit for bit."""
+    a memset; the paced schedule's table is reset by a kernel of the launch itself) and replayed on fresh inputs, with
+    eager work and synchronisation between the replays: every replay must equal the eager result bit for bit."""
     from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
     lens, Hq, Hkv, d, bs, topk = [900, 130, 2000], 32, 2, 128, 64, 8
     q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device)
@@ -177,8 +178,8 @@ def test_forward_backward_replayed_from_a_hip_graph(device):
     sm = d ** -0.5
 
     def step():
-        o, lse = _topk_sparse_attention_fwd(q, k, v, idx, bs, cu, cu, None, None, sm)
-        return (o,) + tuple(_topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, None, None, sm))
+        o, lse = _topk_sparse_attention_fwd(q, k, v, idx, bs, cu, cu, None, None, sm, phases=3 | schedule)
+        return (o,) + tuple(_topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, None, None, sm, phases=7 | schedule))
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
