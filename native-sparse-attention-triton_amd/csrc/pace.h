@@ -11,7 +11,8 @@
 //
 // The pacing is advisory: results do not depend on it.  A wave that has polled `spin_limit` times in one wait stops
 // pacing for the rest of its life, so every wave ends whatever the other waves do (also when fewer workgroups are
-// resident than the launch assumed); a table entry of a wave that has not started or has finished is INT_MAX.
+// resident than the launch assumed); a table entry of a wave that has not started or has finished is INT_MAX; a wave
+// that does not run on the XCD its row stands for does not pace at all.
 #pragma once
 #include "nsa_common.h"
 
@@ -19,7 +20,10 @@
 #define NSA_PACE_MAX_SLOTS 512   // waves per XCD the table has room for
 
 struct PaceParams {
-  int32_t* table;        // [8][NSA_PACE_MAX_SLOTS] int32, then first_sweep[9]: both written by pace_prepare_kernel
+  int32_t* table;        // [8][NSA_PACE_MAX_SLOTS] int32, then first_sweep[9]: both written by pace_prepare_kernel.  The kernels
+                         // take it as an argument of its own (__restrict__): the polls and publishes are atomics, and an
+                         // atomic through a pointer held in a parameter struct makes every array the structs point to a
+                         // possible target, after which none of their uniform loads stays a scalar load
   int slots;             // waves per XCD of this launch (multiple of 4, <= NSA_PACE_MAX_SLOTS)
   int window;            // 64-key units a wave may be ahead of the slowest one
   int spin_limit;        // polls after which a wave gives up pacing
@@ -27,7 +31,7 @@ struct PaceParams {
   int sweeps_per_stream; // ceil(total_len / tokens_per_sweep)
 };
 // XCD x runs the sweeps [first_sweep[x], first_sweep[x + 1]) of the (stream, token) order
-__device__ __host__ __forceinline__ const int32_t* pace_first_sweep(const PaceParams& pp) { return pp.table + 8 * NSA_PACE_MAX_SLOTS; }
+__device__ __host__ __forceinline__ const int32_t* pace_first_sweep(const int32_t* table) { return table + 8 * NSA_PACE_MAX_SLOTS; }
 
 static inline size_t pace_table_bytes() { return (size_t)(8 * NSA_PACE_MAX_SLOTS + 16) * 4; }
 
@@ -109,9 +113,15 @@ struct Pacer {
   int32_t* row;
   int slots, window, spin_limit, me, lane, frontier;
 
-  __device__ __forceinline__ void init(const PaceParams& pp, int xcd, int slot, int lane_) {
-    row = pp.table + xcd * NSA_PACE_MAX_SLOTS;
+  __device__ __forceinline__ void init(const PaceParams& pp, int32_t* table, int xcd, int slot, int lane_) {
+    row = table + xcd * NSA_PACE_MAX_SLOTS;
     slots = pp.slots; window = pp.window; spin_limit = pp.spin_limit; me = slot; lane = lane_; frontier = 0;
+    // The table of a row only works as a meeting point if the row's workgroups share one L2, i.e. if workgroup i runs on
+    // XCD i % 8 (what the hardware's round-robin dispatch gives: measured, all 2048 waves of a launch).  A wave that finds
+    // itself elsewhere does not pace: it would wait on entries it cannot see change.  (A register read, nothing more: an
+    // atomic on the table here made the compiler give up scalar loads in the whole kernel, 2.58 -> 2.75 ms.)
+    const int my_xcc = __builtin_amdgcn_s_getreg(20 /* HW_REG_XCC_ID */ | (0 << 6) | ((4 - 1) << 11));
+    if (my_xcc != xcd) window = NSA_PACE_IDLE;
   }
   // position (in the XCD's running count of 64-key units) of the block this wave turns to next
   __device__ __forceinline__ void publish(int position) {
@@ -154,12 +164,12 @@ struct SweepToken {
 //   visit(tok, who, blk, f)  block blk for the tokens in the bit set who; calls f() once the block's loads are issued;
 //   finish(tok, i, sw)       writes the token's results.
 template <int BS, int TPW, bool AHEAD, typename Tok, typename Ahead, typename Fetch, typename Adopt, typename Visit, typename Finish>
-__device__ __forceinline__ void run_paced_sweeps(const PaceParams& pp, int topk, long long isk, int lane, int slot,
+__device__ __forceinline__ void run_paced_sweeps(const PaceParams& pp, int32_t* table, int topk, long long isk, int lane, int slot,
                                                  Fetch fetch, Adopt adopt, Visit visit, Finish finish) {
   const int xcd = blockIdx.x & 7;
   Pacer pc;
-  pc.init(pp, xcd, slot, lane);
-  const int32_t* first_sweep = pace_first_sweep(pp);
+  pc.init(pp, table, xcd, slot, lane);
+  const int32_t* first_sweep = pace_first_sweep(table);
   const int sw_begin = first_sweep[xcd], sw_end = first_sweep[xcd + 1];
   Ahead ahead[TPW];
   int reach_ahead = 0;

@@ -420,7 +420,7 @@ template <typename T, int D> struct DqToken : SweepToken {
 };
 
 template <typename T, int D, int BS>
-__global__ __launch_bounds__(256) void dq_sweep_kernel(DqParams p, PaceParams pp) {
+__global__ __launch_bounds__(256) void dq_sweep_kernel(DqParams p, PaceParams pp, int32_t* __restrict__ table) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -555,7 +555,7 @@ __global__ __launch_bounds__(256) void dq_sweep_kernel(DqParams p, PaceParams pp
       }
     }
   };
-  run_paced_sweeps<BS, 1, false, Tok, Tok>(pp, p.topk, p.isk, lane, slot, fetch, adopt, visit, finish);
+  run_paced_sweeps<BS, 1, false, Tok, Tok>(pp, table, p.topk, p.isk, lane, slot, fetch, adopt, visit, finish);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -628,7 +628,7 @@ static int run_bwd(const BwdArgs& a) {
       pace.table = (int32_t*)(ws + L.pace);
       pace_fill_params(pace, a.T, pace_slots(), 1, pace_window_units((int)a.D));
       launch_pace_prepare(pace, a.cu, (int)a.B, (int)a.T, GT * (int)a.Hkv, 2000, a.stream);
-      dq_sweep_kernel<T, D, BS><<<(unsigned)(2 * pace.slots), 256, 0, a.stream>>>(p, pace);
+      dq_sweep_kernel<T, D, BS><<<(unsigned)(2 * pace.slots), 256, 0, a.stream>>>(p, pace, pace.table);
     } else {
     long long n_wg = ((p.n_items + 3) / 4 + 7) / 8 * 8;
     if (p.sched.parts) n_wg = 8ll * p.sched.wgs_per_xcd;

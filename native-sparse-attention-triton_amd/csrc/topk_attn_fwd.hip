@@ -301,7 +301,7 @@ __device__ __forceinline__ void fwd_visit_block(FwdToken<T, D> (&tok)[TPW], unsi
 }
 
 template <typename T, int D, int BS, int TPW>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void topk_fwd_sweep_kernel(TopkFwdParams p, PaceParams pp) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void topk_fwd_sweep_kernel(TopkFwdParams p, PaceParams pp, int32_t* __restrict__ table) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (lg == 0) p.lse[(long long)(h * p.G + hq) * p.total_len + k.t] = lsum > 0.f ? k.m * qs + fast_log2(lsum) : -INFINITY;
     }
   };
-  run_paced_sweeps<BS, TPW, TPW == 1, Tok, Ahead>(pp, p.topk, p.isk, lane, slot, fetch, adopt, visit, finish);
+  run_paced_sweeps<BS, TPW, TPW == 1, Tok, Ahead>(pp, table, p.topk, p.isk, lane, slot, fetch, adopt, visit, finish);
 }
 
 // everything one forward call needs on the host side
@@ -388,7 +388,7 @@ static int launch_fwd(const FwdCall& c) {
   if ((c.phases & NSA_FWD_PHASE_ATTEND) && c.pace.slots) {
     launch_pace_prepare(c.pace, p.cu, p.batch, p.total_len, p.GT * p.Hkv, c.fixed_units, c.stream);
     const unsigned n_wg = (unsigned)(2 * c.pace.slots);   // 8 XCDs x slots / 4 workgroups
-    topk_fwd_sweep_kernel<T, D, BS, 1><<<n_wg, 256, 0, c.stream>>>(p, c.pace);
+    topk_fwd_sweep_kernel<T, D, BS, 1><<<n_wg, 256, 0, c.stream>>>(p, c.pace, c.pace.table);
   } else if (c.phases & NSA_FWD_PHASE_ATTEND) {
     long long n_wg = (p.n_items + 3) / 4;
     n_wg = (n_wg + 7) / 8 * 8;

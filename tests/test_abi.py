@@ -27,7 +27,7 @@ def test_version_and_workspace_queries_run_on_host():
     lib = _lib.load()
     assert lib.nsa_version() >= 100
     # size queries are pure host arithmetic
-    # fragment-major copies of K and V, plus the pacing table (8 x 512 entries and the nine sweep bounds, int32)
+    # fragment-major copies of K and V, plus the pacing table (8 x 512 entries  and the nine sweep bounds, int32)
     assert lib.nsa_topk_attn_fwd_workspace_bytes(32768, 1, 4, 128) == 2 * 4 * (1024 + 2) * 128 * 32 * 2 + (8 * 512 + 16) * 4
     assert lib.nsa_topk_attn_bwd_workspace_bytes(2048, 1, 64, 4, 128, 16, 64) > 0
     assert lib.nsa_pool_bwd_workspace_bytes(4095, 2, 32) >= 2 * 64 * 32 * 4
