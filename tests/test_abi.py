@@ -117,6 +117,7 @@ def test_reference_import_paths_resolve():
         "native_sparse_attention.ops.triton.weighted_pool": ["weightedpool_compress", "avgpool_compress"],
         "native_sparse_attention.ops.triton.flash_attention_decode": ["flash_attention_decode"],
         "native_sparse_attention.ops.triton.topk_sparse_attention_decode": ["topk_sparse_attention_decode"],
+        "native_sparse_attention.ops.torch.compressed_attention_decode": ["compressed_attention_decode"],
         "native_sparse_attention.ops.topk_sparse_attention": ["_topk_sparse_attention_fwd", "_topk_sparse_attention_bwd"],
         "native_sparse_attention.ops.compressed_attention": ["_compressed_attention_bwd"],
         "native_sparse_attention.infer": ["nsa_infer"],
