@@ -662,6 +662,86 @@ __global__ __launch_bounds__(256) void cmp_select_kernel(SelParams p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// work items of the dK/dV pass over query ranges (dkdv.h, RANGE = true)
+// chunk_off = exclusive scan of range_chunks over segments (single workgroup).
+static __global__ __launch_bounds__(1024) void chunk_scan_kernel(const int32_t* __restrict__ seg_begin, const int32_t* __restrict__ seg_end, int n_seg,
+                                                          int32_t* __restrict__ chunk_off, int chunk) {
+  __shared__ int part[1024];
+  const int tid = threadIdx.x;
+  const int per = (n_seg + 1023) / 1024;
+  const int j0 = tid * per, j1 = min(n_seg, j0 + per);
+  int s = 0;
+  for (int j = j0; j < j1; j++) s += range_chunks(seg_begin[j], seg_end[j], chunk);
+  part[tid] = s;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    int v = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - s;
+  for (int j = j0; j < j1; j++) {
+    chunk_off[j] = run;
+    run += range_chunks(seg_begin[j], seg_end[j], chunk);
+  }
+  if (tid == 1023) chunk_off[n_seg] = part[1023];
+}
+
+// Launch order of the range-mode work items: by (kv-head, token window), i.e. all key blocks that stream the same
+// `chunk` tokens of Q and dO next to each other.  Together with the contiguous run of the order that each XCD
+// takes (workgroup i runs on XCD i % 8), the workgroups resident on an XCD then read the same rows at about the
+// same time and all but the first find them in its L2; in segment order every work item fetched its rows
+// over the fabric (measured at 65 536 tokens, 32q/2kv heads: 33 GiB of fetches for 1 GiB of Q and dO).
+// Counting sort in one workgroup; the place of an item inside its window is whatever the LDS atomics hand out:
+// it decides when an item runs, not what it computes.  More windows than ORDER_BUCKETS: launch order = item order.
+constexpr int ORDER_BUCKETS = 8192;
+static __global__ __launch_bounds__(1024) void item_order_kernel(const int32_t* __restrict__ seg_begin, const int32_t* __restrict__ chunk_off, int n_seg,
+                                                            int max_blocks, int chunk, int n_win, int32_t* __restrict__ order) {
+  __shared__ int cnt[ORDER_BUCKETS];
+  __shared__ int part[1024];
+  const int tid = threadIdx.x;
+  const int total = chunk_off[n_seg];
+  const int n_bucket = (n_seg / max_blocks) * n_win;
+  if (n_bucket > ORDER_BUCKETS) {
+    for (int i = tid; i < total; i += 1024) order[i] = i;
+    return;
+  }
+  auto bucket_of = [&](int item) {
+    int lo = 0, hi = n_seg;  // chunk_off[lo] <= item < chunk_off[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (chunk_off[mid] <= item) lo = mid; else hi = mid;
+    }
+    return (lo / max_blocks) * n_win + seg_begin[lo] / chunk + (item - chunk_off[lo]);
+  };
+  for (int i = tid; i < n_bucket; i += 1024) cnt[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < total; i += 1024) atomicAdd(&cnt[bucket_of(i)], 1);
+  __syncthreads();
+  const int per = (n_bucket + 1023) / 1024;
+  const int j0 = min(n_bucket, tid * per), j1 = min(n_bucket, j0 + per);
+  int s = 0;
+  for (int j = j0; j < j1; j++) s += cnt[j];
+  part[tid] = s;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int v = tid >= d ? part[tid - d] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - s;
+  for (int j = j0; j < j1; j++) {
+    const int c = cnt[j];
+    cnt[j] = run;  // becomes the bucket's write cursor
+    run += c;
+  }
+  __syncthreads();
+  for (int i = tid; i < total; i += 1024) order[atomicAdd(&cnt[bucket_of(i)], 1)] = i;
+}
+
+// ------------------------------------------------------------------------------------------
 // dK/dV segments: blocks of 64 compressed keys per (head, sequence); their queries are the
 // contiguous range from the first position that sees the block's first key to the sequence end
 __global__ __launch_bounds__(256) void cmp_segments_kernel(const int32_t* __restrict__ cu_q, const int32_t* __restrict__ cu_k, int batch, int Hkv, int ks, int st,

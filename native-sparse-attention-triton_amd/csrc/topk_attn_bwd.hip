@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  constexpr int NK = D / 32, NDT = D / 16, NCH = BS / 32, LD = lds_pitch(D);
+  constexpr int NK = D / 32, NDT = D / 16, LD = lds_pitch(D);
   // K and V come from their fragment-major copies (one coalesced 1 KiB load per operand fragment).
   // Wave-private staging of one 64-key slice of K: the fragments arrive in A-operand layout for
   // S^T = K Q^T, are written through to LDS as rows, and come back transposed (K^T fragments)
