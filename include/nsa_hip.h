@@ -80,9 +80,11 @@ int nsa_topk_attn_fwd(const void* q, const void* k, const void* v, const int32_t
  *     then holds up to 4*Hkv*T*topk entries, and a query appears under the pieces at or before its position.
  * dK/dV are reduced in a fixed order (no atomics): results are run-to-run deterministic.
  * phases: NSA_BWD_PHASE_ALL, or a subset to re-run single passes on a workspace that an
- * earlier call with identical arguments has already filled (PREP = delta + reverse index).
+ * earlier call with identical arguments has already filled (PREP = delta, the (lse, delta) pairs laid out
+ * per token for the dK/dV pass, and the reverse index).
  * When PREP and DQ run in the same call, delta = rowsum(o * dout) is formed inside the dQ pass
- * (which runs before dK/dV) instead of by a pass of its own; the stored values are the same.
+ * (which runs before dK/dV) instead of by a pass of its own (another summation order: the stored values agree to
+ * fp32 rounding).
  * Token strides of q and dout, and group_size * their head strides + D, must fit 31 bits.
  * The dQ pass has the two schedules of the forward (same rule, same bit-identical results);
  * NSA_BWD_SCHEDULE_PLAIN / NSA_BWD_SCHEDULE_PACED or-ed into phases force one of them.

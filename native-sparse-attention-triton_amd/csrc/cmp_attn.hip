@@ -839,7 +839,7 @@ static int run_cmp(CmpArgs& a) {
     item_order_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, chunk_off, n_seg, (int)L.max_blocks, L.chunk, (int)(a.Tq / L.chunk + 1), order);
     DkdvParams d;
     d.order = order;
-    d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
+    d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.stat = nullptr; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
     d.cu_blk = cu_blk; d.seg_begin = seg_begin; d.seg_end = seg_end; d.chunk_off = chunk_off; d.queries = nullptr;
     d.partial = (float*)(a.ws + L.partial);
     d.total_len = (int)a.Tq; d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;

@@ -47,6 +47,9 @@ __device__ __forceinline__ int range_chunks(int begin, int end, int chunk) { ret
 
 struct DkdvParams {
   const void* q; const void* k; const void* v; const void* dout; const float* lse; const float* delta;
+  // list mode: (lse, delta) pairs per token, [total_len][Hkv * G][2].  A work item's tokens are scattered, and in the [head][token] arrays
+  // above the 16 heads of a token lie in 32 different cache lines (39 % of the pass's L2 requests went there); here they share one.
+  const float* stat;
   const int32_t* cu; const int32_t* cu_k; const int32_t* cu_blk; const int32_t* seg_begin; const int32_t* seg_end; const int32_t* chunk_off; const int32_t* queries;
   const int32_t* order;  // range mode: launch order of the work items (item_order_kernel), or null
   float* partial;
@@ -190,7 +193,8 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS == 64 ? (GT1 ? 3 : 2) : (BS
       const int r = min(step * 2 + rg, n_rg - 1);
       const int t = tok_s[GT1 ? r : r / GT];
       const int hq = min((GT1 ? 0 : (r % GT) * 16) + hd, p.G - 1);
-      dma4((lane < 32 ? lbase : ebase) + (long long)hq * p.total_len + t, buf + 2 * TENSOR_BYTES);
+      if (RANGE) dma4((lane < 32 ? lbase : ebase) + (long long)hq * p.total_len + t, buf + 2 * TENSOR_BYTES);
+      else dma4(p.stat + (((long long)t * p.Hkv + h) * p.G + hq) * 2 + (lane >> 5), buf + 2 * TENSOR_BYTES);
     }
   };
 

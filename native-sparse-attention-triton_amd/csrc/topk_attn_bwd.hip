@@ -24,7 +24,7 @@
 // ------------------------------------------------------------------------------------------
 // workspace carving (host and entry point must agree)
 struct BwdLayout {
-  size_t delta, cu_blk, hist, queries, seg_off, chunk_off, kf, vf, pace, partial, total;
+  size_t delta, stat, cu_blk, hist, queries, seg_off, chunk_off, kf, vf, pace, partial, total;
   int64_t max_blocks, n_pairs, max_items, n_slots;
   int tile_tokens, n_tiles;
 };
@@ -54,6 +54,7 @@ static BwdLayout bwd_layout(int64_t T, int64_t B, int64_t Hq, int64_t Hkv, int64
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += align256(bytes); return o; };
   L.delta = take((size_t)Hq * T * 4);
+  L.stat = take((size_t)Hq * T * 8);   // (lse, delta) per token and head, token-major
   L.cu_blk = take((size_t)(B + 1) * 4);
   L.hist = take((size_t)Hkv * L.n_tiles * L.max_blocks * 4);   // [head][tile][block] counts, then their prefix over tiles
   L.queries = take((size_t)L.n_pairs * 4);
@@ -252,6 +253,7 @@ struct DqParams {
   const void* q; const void* kf; const void* vf; const void* dout; const float* lse;
   const void* o;   // forward output: when given, delta = rowsum(O * dO) is formed here and stored for the dK/dV pass
   float* delta;    // read when o is null
+  float* stat;     // (lse, delta) of every row, [total_len][Hq][2]: written for the dK/dV pass
   const int32_t* idx; const int32_t* cu; void* dq;
   int total_len, batch, Hkv, G, GT, topk, n_slots;
   long long n_items;
@@ -321,6 +323,7 @@ __global__ __launch_bounds__(256) void dq_kernel(DqParams p) {
   } else {
     dl = has_head ? p.delta[(long long)hh * p.total_len + t] : 0.f;
   }
+  if (has_head && lg == 0) *reinterpret_cast<float2*>(p.stat + ((long long)t * p.Hkv * p.G + hh) * 2) = float2{l2, dl};
   f32x4 acc[NDT];
 #pragma unroll
   for (int i = 0; i < NDT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -478,6 +481,7 @@ __global__ __launch_bounds__(256) void dq_sweep_kernel(DqParams p, PaceParams pp
     } else {
       dl = has_head ? p.delta[(long long)hh * p.total_len + t] : 0.f;
     }
+    if (has_head && lg == 0) *reinterpret_cast<float2*>(p.stat + ((long long)t * p.Hkv * p.G + hh) * 2) = float2{k.l2, dl};
     k.dls = dl * p.sm_scale;
     k.todo = __ballot(k.my_blk >= 0 && k.my_blk <= k.qb);
   };
@@ -600,7 +604,7 @@ static int run_bwd(const BwdArgs& a) {
   // rows anyway), by a pass of its own when only the preparation is asked for
   const bool fused_delta = (a.phases & NSA_BWD_PHASE_PREP) && (a.phases & NSA_BWD_PHASE_DQ);
   if ((a.phases & NSA_BWD_PHASE_PREP) && !fused_delta)
-    launch_delta<T, D>((const T*)a.o, (const T*)a.dout, delta, a.T, a.Hq, a.osn, a.osh, a.dsn, a.dsh, a.stream);
+    launch_delta<T, D>((const T*)a.o, (const T*)a.dout, delta, a.T, a.Hq, a.osn, a.osh, a.dsn, a.dsh, a.stream, a.lse, (float*)(ws + L.stat));
   if (a.phases & NSA_BWD_PHASE_PREP) {
     int rc = build_reverse_index(a, L);
     if (rc != NSA_OK) return rc;
@@ -615,7 +619,7 @@ static int run_bwd(const BwdArgs& a) {
     T* kf = (T*)(ws + L.kf);
     T* vf = (T*)(ws + L.vf);
     launch_retile_pair<T, D, RETILE_ROWS, RETILE_ROWS>((const T*)a.k, kf, a.ksn, a.ksh, (const T*)a.v, vf, a.vsn, a.vsh, a.cu, a.B, L.n_slots, a.Hkv, a.stream);
-    p.q = a.q; p.kf = kf; p.vf = vf; p.dout = a.dout; p.lse = a.lse; p.o = fused_delta ? a.o : nullptr; p.delta = delta; p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
+    p.q = a.q; p.kf = kf; p.vf = vf; p.dout = a.dout; p.lse = a.lse; p.o = fused_delta ? a.o : nullptr; p.delta = delta; p.stat = (float*)(ws + L.stat); p.idx = a.idx; p.cu = a.cu; p.dq = a.dq;
     p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.topk = (int)a.topk; p.n_slots = (int)L.n_slots;
     p.n_items = (long long)a.T * GT * a.Hkv;
     p.qsn = a.qsn; p.qsh = a.qsh; p.dsn = a.dsn; p.dsh = a.dsh; p.osn = a.osn; p.osh = a.osh;
@@ -638,7 +642,7 @@ static int run_bwd(const BwdArgs& a) {
   if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;
     p.order = nullptr;
-    p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.cu = a.cu;
+    p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.stat = (const float*)(ws + L.stat); p.cu = a.cu;
     p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_begin = (const int32_t*)(ws + L.seg_off); p.seg_end = p.seg_begin + 1;
     p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.queries);
     p.partial = (float*)(ws + L.partial);

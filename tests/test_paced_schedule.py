@@ -71,3 +71,29 @@ def test_paced_negative_and_zero_scale(device):
         assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]), sm
         want = oracle.topk_sparse_attention(q.float(), k.float(), v.float(), idx, 64, cu, softmax_scale=sm)
         assert_close(b[0], want, "o at scale %g" % sm)
+
+
+def test_passes_one_call_at_a_time(device):
+    """The backward's passes run as separate calls on a kept workspace: preparation alone forms delta and the per-token
+    (lse, delta) pairs in a pass of its own (a different summation order from the one inside the dQ pass, so the last
+    bits of delta may differ from the single call's); dK/dV before or after dQ gives identical results."""
+    from native_sparse_attention import _lib
+    lens, Hq, Hkv, d, bs, topk = [900, 2300, 70], 32, 2, 128, 64, 8
+    q, k, v, do, cu = _inputs(lens, Hq, Hkv, d, torch.bfloat16, device)
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=6)
+    n, sm = max(lens), d ** -0.5
+    o, lse = _topk_sparse_attention_fwd(q, k, v, idx, bs, cu, cu, n, n, sm)
+    want = _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, n, n, sm)
+    lib = _lib.load()
+    got = []
+    for order in ((1, 4, 2), (1, 2, 4)):
+        ws = _lib.workspace(lib.nsa_topk_attn_bwd_workspace_bytes(sum(lens), len(lens), Hq, Hkv, d, topk, bs), device)
+        ws.fill_(0x7f)   # nothing may be read before a pass has written it
+        out = tuple(torch.full_like(x, float("nan")) for x in want)
+        for phase in order:
+            _topk_sparse_attention_bwd(o, do, lse, q, k, v, idx, bs, cu, cu, n, n, sm, workspace=ws, phases=phase, out=out)
+        torch.cuda.synchronize()
+        got.append(out)
+    for name, a, b, c in zip(("dq", "dk", "dv"), want, got[0], got[1]):
+        assert torch.equal(b, c), name + " depends on the order of the passes"
+        assert_close(b, a.float(), name + " (separate passes)", rel_to=True)
