@@ -28,7 +28,7 @@ HQ, HKV, D, BS = 64, 4, 128, 64
 H100_FWD_BWD_MS = 12.417 + 15.154
 # memory-side traffic per launch at the default workload (N=32768, top16), bytes: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, scaled by what the same counters read for a plain 1 GiB copy (x2.0 and x1.0); see profiles/
-MEASURED_TRAFFIC = {"topk_fwd_sweep_kernel": 8.54 * 2**30, "dq_sweep_kernel": 9.76 * 2**30, "dkdv_kernel": 18.28 * 2**30}
+MEASURED_TRAFFIC = {"topk_fwd_sweep_kernel": 8.38 * 2**30, "dq_sweep_kernel": 9.71 * 2**30, "dkdv_kernel": 16.15 * 2**30}
 
 
 def _paced(N, topk):
