@@ -20,6 +20,7 @@
 struct CmpParams {
   const void* q; const void* k; const void* v; const void* dout; void* o; void* dq; float* lse; const float* delta;
   float* delta_out;  // backward dQ: when set, delta = rowsum(o * dout) is formed there (from the dO rows it holds) and stored here
+  float* stat_out;   // backward dQ: (lse, delta) of every row, token-major [total_q][Hkv * G][2], for the dK/dV pass
   const int32_t* cu_q; const int32_t* cu_k;
   int total_q, batch, Hkv, G, GT, ks, st;
   int window;  // -1: compressed keys (rule above); >= 0: ordinary keys, position i sees j in [i - window, i]; -2: ordinary keys, all visible
@@ -363,6 +364,7 @@ __global__ __launch_bounds__(256) void cmp_dq_kernel(CmpParams p) {
     } else {
       dl[j] = live ? p.delta[(long long)hh * p.total_q + t] : 0.f;
     }
+    if (p.stat_out && live && lg == 0) *reinterpret_cast<float2*>(p.stat_out + (t * p.Hkv * p.G + hh) * 2) = float2{l2[j], dl[j]};
   }
   int tile_lo, tile_hi, unused;
   visible_range(min(ti.i0 + 7, ti.lq - 1), ti.lq, ti.lk, p.ks, p.st, p.window, unused, tile_hi);
@@ -768,7 +770,7 @@ __global__ __launch_bounds__(256) void cmp_segments_kernel(const int32_t* __rest
   }
 }
 
-struct CmpBwdLayout { size_t delta, cu_blk, seg_begin, seg_end, chunk_off, order, partial, total; int64_t max_blocks, max_items; int chunk; };
+struct CmpBwdLayout { size_t delta, stat, cu_blk, seg_begin, seg_end, chunk_off, order, partial, total; int64_t max_blocks, max_items; int chunk; };
 static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
   CmpBwdLayout L;
   L.max_blocks = Tk / 64 + B;
@@ -779,6 +781,7 @@ static CmpBwdLayout cmp_bwd_layout(int64_t Tq, int64_t Tk, int64_t B, int64_t Hq
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
   L.delta = take((size_t)Hq * Tq * 4);
+  L.stat = take((size_t)Hq * Tq * 8);
   L.cu_blk = take((size_t)(B + 1) * 4);
   L.seg_begin = take((size_t)(Hkv * L.max_blocks + 1) * 4);
   L.seg_end = take((size_t)(Hkv * L.max_blocks + 1) * 4);
@@ -831,7 +834,7 @@ static int run_cmp(CmpArgs& a) {
     int32_t* chunk_off = (int32_t*)(a.ws + L.chunk_off);
     const int n_seg = (int)(a.Hkv * L.max_blocks);
     // dQ first: it forms delta = rowsum(O * dO) from the dO rows it holds and leaves it behind for the dK/dV pass
-    a.p.o = const_cast<void*>(a.o_in); a.p.delta = nullptr; a.p.delta_out = delta;
+    a.p.o = const_cast<void*>(a.o_in); a.p.delta = nullptr; a.p.delta_out = delta; a.p.stat_out = (float*)(a.ws + L.stat);
     cmp_dq_kernel<T, D><<<dim3((unsigned)(2 * slots), (unsigned)(a.Hkv * a.p.GT)), 256, 0, a.stream>>>(a.p);
     cmp_segments_kernel<<<1, 256, (size_t)(a.B + 1) * 4, a.stream>>>(a.p.cu_q, a.p.cu_k, (int)a.B, (int)a.Hkv, a.p.ks, a.p.st, a.p.window, (int)L.max_blocks, cu_blk, seg_begin, seg_end);
     chunk_scan_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, seg_end, n_seg, chunk_off, L.chunk);
@@ -839,10 +842,10 @@ static int run_cmp(CmpArgs& a) {
     item_order_kernel<<<1, 1024, 0, a.stream>>>(seg_begin, chunk_off, n_seg, (int)L.max_blocks, L.chunk, (int)(a.Tq / L.chunk + 1), order);
     DkdvParams d;
     d.order = order;
-    d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.lse = a.p.lse; d.delta = delta; d.stat = nullptr; d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
+    d.q = a.p.q; d.k = a.p.k; d.v = a.p.v; d.dout = a.p.dout; d.stat = (const float*)(a.ws + L.stat); d.cu = a.p.cu_q; d.cu_k = a.p.cu_k;
     d.cu_blk = cu_blk; d.seg_begin = seg_begin; d.seg_end = seg_end; d.chunk_off = chunk_off; d.queries = nullptr;
     d.partial = (float*)(a.ws + L.partial);
-    d.total_len = (int)a.Tq; d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;
+    d.batch = (int)a.B; d.Hkv = (int)a.Hkv; d.G = a.p.G; d.GT = a.p.GT; d.max_blocks = (int)L.max_blocks;
     d.n_seg = n_seg; d.ks = a.p.ks; d.st = a.p.st; d.window = a.p.window; d.chunk = L.chunk;
     d.qsn = (int)a.p.qsn; d.qsh = (int)a.p.qsh; d.ksn = a.p.ksn; d.ksh = a.p.ksh; d.vsn = a.p.vsn; d.vsh = a.p.vsh; d.dsn = (int)a.p.dsn; d.dsh = (int)a.p.dsh;
     d.qk_scale = a.p.qk_scale; d.sm_scale = a.p.sm_scale;
@@ -880,7 +883,7 @@ static int cmp_common(CmpArgs& a, const void* q, const void* k, const void* v, c
   p.qsn = strides[0]; p.qsh = strides[1]; p.ksn = strides[2]; p.ksh = strides[3]; p.vsn = strides[4]; p.vsh = strides[5];
   // forward: a zero scale is applied as the smallest positive one (masked scores are -inf there, and 0 * inf has no value)
   p.qk_scale = (sm_scale == 0.f ? 1.17549435e-38f : sm_scale) * NSA_LOG2E; p.sm_scale = sm_scale; p.window = -1;
-  p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr; p.delta_out = nullptr;
+  p.dout = nullptr; p.o = nullptr; p.dq = nullptr; p.lse = nullptr; p.delta = nullptr; p.delta_out = nullptr; p.stat_out = nullptr;
   a.Tq = Tq; a.Tk = Tk; a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.stream = (hipStream_t)stream; a.ws = nullptr;
   return NSA_OK;
 }

@@ -46,14 +46,15 @@ constexpr int dkdv_waves(int bs) { return bs >= 256 ? 8 : (bs >= 64 ? 4 : bs / 1
 __device__ __forceinline__ int range_chunks(int begin, int end, int chunk) { return end > begin ? (end + chunk - 1) / chunk - begin / chunk : 0; }
 
 struct DkdvParams {
-  const void* q; const void* k; const void* v; const void* dout; const float* lse; const float* delta;
-  // list mode: (lse, delta) pairs per token, [total_len][Hkv * G][2].  A work item's tokens are scattered, and in the [head][token] arrays
-  // above the 16 heads of a token lie in 32 different cache lines (39 % of the pass's L2 requests went there); here they share one.
+  const void* q; const void* k; const void* v; const void* dout;
+  // (lse, delta) pairs per token, [tokens][Hkv * G][2], left behind by the dQ pass (or the stand-alone delta pass).  In [head][token]
+  // arrays the 16 heads of a token lie in 32 different cache lines: with the scattered tokens of a query list 39 % of the pass's
+  // L2 requests went there; here they share one line.
   const float* stat;
   const int32_t* cu; const int32_t* cu_k; const int32_t* cu_blk; const int32_t* seg_begin; const int32_t* seg_end; const int32_t* chunk_off; const int32_t* queries;
   const int32_t* order;  // range mode: launch order of the work items (item_order_kernel), or null
   float* partial;
-  int total_len, batch, Hkv, G, GT, max_blocks, n_seg, ks, st;
+  int batch, Hkv, G, GT, max_blocks, n_seg, ks, st;
   int chunk;   // queries per work item (dkdv_chunk_tokens)
   int window;  // range mode: -1 compressed keys (key c seen from position c*st + ks - 1 on), >= 0 ordinary keys seen by [key, key + window], -2 every key seen by every position
   long long ksn, ksh, vsn, vsh;
@@ -161,8 +162,6 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS == 64 ? (GT1 ? 3 : 2) : (BS
 
   const T* const qbase = (const T*)p.q + (long long)h * p.G * p.qsh;
   const T* const dbase = (const T*)p.dout + (long long)h * p.G * p.dsh;
-  const float* const lbase = p.lse + (long long)h * p.G * p.total_len;
-  const float* const ebase = p.delta + (long long)h * p.G * p.total_len;
 
   constexpr int NI = CP / 2;                 // 1 KiB wave-copies per tensor per step
   constexpr int LPW = (NI + NW - 1) / NW;    // of which one wave issues at most this many
@@ -193,8 +192,7 @@ __global__ __launch_bounds__(64 * dkdv_waves(BS), BS == 64 ? (GT1 ? 3 : 2) : (BS
       const int r = min(step * 2 + rg, n_rg - 1);
       const int t = tok_s[GT1 ? r : r / GT];
       const int hq = min((GT1 ? 0 : (r % GT) * 16) + hd, p.G - 1);
-      if (RANGE) dma4((lane < 32 ? lbase : ebase) + (long long)hq * p.total_len + t, buf + 2 * TENSOR_BYTES);
-      else dma4(p.stat + (((long long)t * p.Hkv + h) * p.G + hq) * 2 + (lane >> 5), buf + 2 * TENSOR_BYTES);
+      dma4(p.stat + (((long long)t * p.Hkv + h) * p.G + hq) * 2 + (lane >> 5), buf + 2 * TENSOR_BYTES);
     }
   };
 

@@ -642,11 +642,11 @@ static int run_bwd(const BwdArgs& a) {
   if (a.phases & NSA_BWD_PHASE_DKDV) {
     DkdvParams p;
     p.order = nullptr;
-    p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.lse = a.lse; p.delta = delta; p.stat = (const float*)(ws + L.stat); p.cu = a.cu;
+    p.q = a.q; p.k = a.k; p.v = a.v; p.dout = a.dout; p.stat = (const float*)(ws + L.stat); p.cu = a.cu;
     p.cu_blk = (const int32_t*)(ws + L.cu_blk); p.seg_begin = (const int32_t*)(ws + L.seg_off); p.seg_end = p.seg_begin + 1;
     p.chunk_off = (const int32_t*)(ws + L.chunk_off); p.queries = (const int32_t*)(ws + L.queries);
     p.partial = (float*)(ws + L.partial);
-    p.total_len = (int)a.T; p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
+    p.batch = (int)a.B; p.Hkv = (int)a.Hkv; p.G = G; p.GT = GT; p.max_blocks = (int)L.max_blocks; p.n_seg = n_seg;
     p.qsn = (int)a.qsn; p.qsh = (int)a.qsh; p.ksn = a.ksn; p.ksh = a.ksh; p.vsn = a.vsn; p.vsh = a.vsh; p.dsn = (int)a.dsn; p.dsh = (int)a.dsh;
     p.qk_scale = a.sm_scale * NSA_LOG2E; p.sm_scale = a.sm_scale; p.cu_k = a.cu; p.ks = 1; p.st = 1; p.window = -1;
     p.chunk = dkdv_chunk_tokens(L.n_pairs, LIST_CHUNK);
