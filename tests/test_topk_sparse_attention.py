@@ -120,6 +120,49 @@ def test_repeated_block_ids_count_once(device, schedule):
         assert_close(got, ref, name, rel_to=ref.abs().max().item())
 
 
+@pytest.mark.parametrize("schedule", [8, 16])   # NSA_*_SCHEDULE_PLAIN / _PACED
+def test_rows_that_select_nothing(device, schedule):
+    """Tokens whose row holds no block they may see (all -1, or only blocks after their own) get a zero output, lse = -inf
+    and zero gradients, and change nothing for the other tokens.  (The reference's generator always lists block 0; its
+    kernel divides 0 by 0 for such a row.)"""
+    from native_sparse_attention.ops.topk_sparse_attention import _topk_sparse_attention_bwd, _topk_sparse_attention_fwd
+
+    lens, Hq, Hkv, d, bs, topk = [1100, 700], 16, 2, 128, 64, 5
+    q, k, v, cu = _make(lens, Hq, Hkv, d, torch.bfloat16, device, seed=5)
+    idx = make_topk_idx(cu, bs, topk, Hkv, seed=9)
+    T = q.shape[0]
+    g = torch.Generator(device=device).manual_seed(12)
+    do = torch.randn(q.shape, generator=g, device=device).to(q.dtype)
+    empty = torch.zeros(Hkv, T, dtype=torch.bool, device=device)
+    empty[0, 5::7] = True
+    empty[1, 3::11] = True
+    empty[:, :3] = True
+    gone = idx.clone()
+    gone[empty] = -1
+    gone[0, 12::14] = 10_000                       # blocks far after the token's own: skipped like -1
+    empty[0, 12::14] = True
+    n, sm = max(lens), d ** -0.5
+    o, lse = _topk_sparse_attention_fwd(q, k, v, gone, bs, cu, cu, n, n, sm, phases=3 | schedule)
+    dq, dk, dv = _topk_sparse_attention_bwd(o, do, lse, q, k, v, gone, bs, cu, cu, n, n, sm, phases=7 | schedule)
+    torch.cuda.synchronize()
+    rows = empty.repeat_interleave(Hq // Hkv, 0)   # [Hq, T]
+    assert (o.transpose(0, 1)[rows] == 0).all() and (dq.transpose(0, 1)[rows] == 0).all()
+    assert (lse[rows] == float("-inf")).all()
+    for x in (o, dq, dk, dv):
+        assert torch.isfinite(x.float()).all()
+    # the other tokens: the oracle on the original ids, with the emptied rows' dO zeroed so that they add nothing to dK / dV
+    do_ref = do.float().clone()
+    do_ref.transpose(0, 1)[rows] = 0
+    qf, kf, vf = (x.float().requires_grad_() for x in (q, k, v))
+    want = oracle.topk_sparse_attention(qf, kf, vf, idx, bs, cu)
+    want.backward(do_ref)
+    keep = ~rows
+    assert_close(o.transpose(0, 1)[keep], want.detach().transpose(0, 1)[keep], "o of the other rows")
+    assert_close(dq.transpose(0, 1)[keep], qf.grad.transpose(0, 1)[keep], "dq of the other rows", rel_to=qf.grad.abs().max().item())
+    assert_close(dk, kf.grad, "dk", rel_to=kf.grad.abs().max().item())
+    assert_close(dv, vf.grad, "dv", rel_to=vf.grad.abs().max().item())
+
+
 def _expand_to_pieces(idx, cu, bs, piece):
     """Ids of the `piece`-key pieces of the selected bs-key blocks that start at or before each token (-1 elsewhere)."""
     sub = bs // piece
